@@ -1,0 +1,201 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-prefix decode attention hot path on one MI355X.
+
+Workload (BASELINE.json configs[2], "C3"): one denoise step = the attention of all 28 layers for 8
+requests, each with 128 query + 32 response rows (Dream-7B GQA 28/4, d=128, bf16) over its
+top-K = 8 of 32 chunks compacted to 512 tokens (16 non-contiguous 256-token pages per request out
+of a shared, seeded page pool) plus the active block itself.  The prefix KV stays fixed over the
+steps.  Inputs are synthetic (N(0,1)/sqrt(128)) and resident in HBM before the timed region.
+
+Prints ONE JSON line: metric = microseconds per denoise step (lower is better), with the roofline
+of the dominant kernel (attn_fwd_kernel) and the CPU oracle timed on a bounded sample next to it.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
+PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
+
+HQ, HKV, D, PAGE = 28, 4, 128, 256
+LAYERS, N_REQ, N_CHUNKS, TOPK, CHUNK_TOKENS = 28, 8, 32, 8, 512
+Q_LEN = 160
+
+
+def build_workload(torch, dev, q_len=Q_LEN, layers=LAYERS, n_req=N_REQ, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    pages_per_req = N_CHUNKS * CHUNK_TOKENS // PAGE            # logical pages of a request's prefix
+    sel_pages = TOPK * CHUNK_TOKENS // PAGE                    # 16 pages actually read
+    n_pages = n_req * pages_per_req + 1
+    std = 1.0 / math.sqrt(D)
+    gd = torch.Generator(device=dev).manual_seed(seed)
+    kv = torch.empty((2, layers, n_pages, PAGE, HKV, D), dtype=torch.bfloat16, device=dev)
+    for l in range(layers):  # fill per layer to bound the fp32 temporary
+        kv[:, l] = (torch.randn((2, n_pages, PAGE, HKV, D), generator=gd, device=dev) * std).to(torch.bfloat16)
+    perm = torch.randperm(n_pages, generator=g)
+    block_table = torch.stack([perm[r * pages_per_req:(r + 1) * pages_per_req] for r in range(n_req)]).to(torch.int32)
+    ptr, start, length = [0], [], []
+    for r in range(n_req):
+        sel = sorted(torch.randperm(N_CHUNKS, generator=g)[:TOPK].tolist())
+        for c in sel:
+            start.append(c * CHUNK_TOKENS)
+            length.append(CHUNK_TOKENS)
+        ptr.append(len(start))
+    mk = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    n_tok = n_req * q_len
+    q = (torch.randn((layers, n_tok, HQ, D), generator=gd, device=dev) * std).to(torch.bfloat16)
+    kn = (torch.randn((layers, n_tok, HKV, D), generator=gd, device=dev) * std).to(torch.bfloat16)
+    vn = (torch.randn((layers, n_tok, HKV, D), generator=gd, device=dev) * std).to(torch.bfloat16)
+    out = torch.empty_like(q)
+    qsl = torch.arange(0, n_tok + 1, q_len, dtype=torch.int32, device=dev)
+    return dict(kv=kv, block_table=block_table.to(dev), ranges=(mk(ptr), mk(start), mk(length), TOPK), q=q, kn=kn,
+                vn=vn, out=out, qsl=qsl, q_len=q_len, ctx=TOPK * CHUNK_TOKENS, n_req=n_req, layers=layers,
+                ranges_host=[[(start[i], length[i]) for i in range(ptr[r], ptr[r + 1])] for r in range(n_req)],
+                sel_pages=sel_pages)
+
+
+def algorithmic_work(q_len, ctx, n_req):
+    """Per launch (= one layer, all requests): bytes and FLOPs of SURVEY section 8(d)."""
+    by = n_req * (2 * ctx * HKV * D * 2 + 2 * q_len * HKV * D * 2 + 2 * q_len * HQ * D * 2)
+    fl = n_req * 4 * q_len * (ctx + q_len) * D * HQ
+    return by, fl
+
+
+def prepare(ops, w, rows_per_group=0, num_splits=0):
+    preps = []
+    for l in range(w["layers"]):
+        preps.append(ops.PreparedAttention(w["q"][l], w["kn"][l], w["vn"][l], w["kv"][0, l], w["kv"][1, l],
+                                           w["block_table"], w["qsl"], max_q_len=w["q_len"], max_ctx_len=w["ctx"],
+                                           ranges=w["ranges"], out=w["out"][l], rows_per_group=rows_per_group,
+                                           num_splits=num_splits))
+    return preps
+
+
+def time_steps(torch, preps, steps, warmup):
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(warmup):
+        for p in preps:
+            p.run(stream)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        for p in preps:
+            p.run(stream)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, e0.elapsed_time(e1) * 1e-3
+
+
+def cpu_baseline(torch, w, sample_layers=1):
+    """The CPU oracle (a PyTorch restatement of the reference path: page-table gather + fp32
+    masked softmax attention with GQA repeat) on `sample_layers` layer(s) of the same workload."""
+    from oracle import ref_ops
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    l = 0
+    args = [w[k][l].cpu() for k in ("q", "kn", "vn")]
+    kc, vc = w["kv"][0, l].cpu(), w["kv"][1, l].cpu()
+    bt, qsl = w["block_table"].cpu(), w["qsl"].cpu()
+    ref_ops.sparse_decode_attention(*args, kc, vc, bt, qsl, w["ranges_host"])  # warm-up
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for _ in range(sample_layers):
+            ref = ref_ops.sparse_decode_attention(*args, kc, vc, bt, qsl, w["ranges_host"])
+        times.append(time.perf_counter() - t0)
+    per_layer = sorted(times)[1] / sample_layers
+    return per_layer, cores, ref
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=32)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--rows-per-group", type=int, default=0, help="override the row-group size (tuning)")
+    ap.add_argument("--num-splits", type=int, default=0, help="override the KV split count (tuning)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the secondary shapes")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build is single-GPU (one MI355X); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from prefilling_dllm_amd import ops
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    w = build_workload(torch, dev)
+    preps = prepare(ops, w, args.rows_per_group, args.num_splits)
+    wall, gpu_s = time_steps(torch, preps, args.steps, args.warmup)
+    launches = args.steps * w["layers"]
+    us_per_step = gpu_s / args.steps * 1e6
+    launch_s = gpu_s / launches
+    by, fl = algorithmic_work(w["q_len"], w["ctx"], w["n_req"])
+    tflops = fl / launch_s / 1e12
+    gbs = by / launch_s / 1e9
+
+    # parity spot check of the timed outputs against the oracle (layer 0), and the CPU baseline
+    cpu = None
+    if not args.no_cpu:
+        per_layer, cores, ref = cpu_baseline(torch, w)
+        err = (w["out"][0].float().cpu() - ref).abs().max().item()
+        if not err <= 2e-2:
+            print(f"bench.py: parity check failed, max abs err {err}", file=sys.stderr)
+            sys.exit(4)
+        cpu = {"value": per_layer * w["layers"] * 1e6, "unit": "us/step", "cores": cores, "kind": "port",
+               "sample": f"1 of {w['layers']} layers x {w['n_req']} requests of the same step (median of 3), "
+                         f"extrapolated x{w['layers']}", "max_abs_err_vs_gpu": err}
+
+    extras = {}
+    if not args.no_extras:
+        # response-only block (the reference engine's real decode shape, 32 rows): the HBM-bound case
+        w32 = build_workload(torch, dev, q_len=32, layers=4)
+        p32 = prepare(ops, w32)
+        _, g32 = time_steps(torch, p32, 16, 2)
+        b32, f32_ = algorithmic_work(32, w32["ctx"], w32["n_req"])
+        l32 = g32 / (16 * 4)
+        extras["decode_32_rows"] = {"us_per_launch": l32 * 1e6, "us_per_step_28_layers": l32 * 28e6,
+                                    "hbm_GBps": b32 / l32 / 1e9, "hbm_frac": b32 / l32 / 1e9 / PEAK_HBM_GBS,
+                                    "bf16_TFLOPs": f32_ / l32 / 1e12}
+        del w32, p32
+
+    rows, splits = ops.attention_plan(w["n_req"], HQ, HKV, max_q_len=w["q_len"], max_ctx_len=w["ctx"],
+                                      num_splits=args.num_splits, rows_per_group=args.rows_per_group)
+    line = {
+        "metric": "us/denoise-step sparse-KV attention, 32K prefix top-K=8 (28 layers, 8 requests, 160 rows)",
+        "value": us_per_step, "unit": "us/step", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": us_per_step / 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[2]: 28-layer sparse-prefix decode step, 8 req x (128 query + 32 "
+                               "response rows) over 8x512 non-contiguous KV tokens in 256-token pages, GQA 28/4 d128",
+                   "rows_per_workgroup": rows, "kv_splits": splits},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "attn_fwd_kernel", "avg_launch_us": launch_s * 1e6,
+                     "algorithmic_flops_per_launch": fl, "algorithmic_bytes_per_launch": by},
+        "hbm": {"achieved_GBps": gbs, "peak_GBps": PEAK_HBM_GBS, "frac": gbs / PEAK_HBM_GBS},
+        "cpu_baseline": cpu,
+        "wall_s_timed_region": wall,
+        "extras": extras,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,291 @@
+/*
+ * pdllm.h -- C ABI of the MI355X (gfx950) hot path of Prefilling-dLLM.
+ *
+ * Every entry point takes plain device pointers, sizes and strides, launches on
+ * the given HIP stream and returns an int status (PDLLM_OK or a negative
+ * PDLLM_ERR_* code).  Nothing here allocates, frees or synchronises; scratch
+ * memory is a caller-provided workspace whose size a *_workspace_bytes query
+ * returns.  No entry point throws across the boundary.
+ *
+ * Each declaration cites the reference interface it replaces.  Paths are
+ * relative to prefilling_dllm_engine/prefilling_dllm/ of the reference:
+ *   OPS = layers/attention/ops,  ENG = fastdllm_engine.py
+ */
+#ifndef PDLLM_H
+#define PDLLM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* pdllm_stream_t; /* a hipStream_t (0 = the null stream) */
+
+enum {
+  PDLLM_OK = 0,
+  PDLLM_ERR_NULL = -1,        /* a required pointer is NULL                       */
+  PDLLM_ERR_SHAPE = -2,       /* a size is negative / inconsistent / unsupported  */
+  PDLLM_ERR_STRIDE = -3,      /* a stride or alignment the kernels rely on fails  */
+  PDLLM_ERR_DTYPE = -4,       /* unknown dtype / mode enumerator                  */
+  PDLLM_ERR_WORKSPACE = -5,   /* workspace missing or too small                   */
+  PDLLM_ERR_LAUNCH = -6,      /* hipLaunch reported an error                      */
+  PDLLM_ERR_UNSUPPORTED = -7  /* valid request the kernels do not cover           */
+};
+
+enum { PDLLM_KV_BF16 = 0, PDLLM_KV_FP8_E4M3 = 1 };
+/* visibility of the in-flight (active) keys; cached prefix keys are always visible */
+enum { PDLLM_MASK_FULL = 0, PDLLM_MASK_CAUSAL = 1, PDLLM_MASK_DENSE = 2 };
+
+const char* pdllm_status_string(int status);
+/* version of this ABI; bumped when a struct layout changes */
+int pdllm_abi_version(void);
+
+/* ------------------------------------------------------------------------- *
+ * Paged KV store                                                             *
+ * ------------------------------------------------------------------------- */
+
+/* Replaces store_kvcache_unified_layout + store_kvcache_kernel_diffusion_lm
+ * (OPS/kv_cache_kernels.py:150-172, 34-55).
+ * key/value: [n_tokens, Hkv*d] rows of row_elems 16-bit elements, row strides
+ * key_stride / value_stride (elements).  k_cache/v_cache viewed as
+ * [n_slots, row_elems].  slot_mapping[n_tokens] int32; slot < 0 = skip the
+ * token; slot >= n_slots is skipped as well (never written out of bounds). */
+int pdllm_kv_store(const void* key, const void* value, void* k_cache, void* v_cache,
+                   const int32_t* slot_mapping, int64_t n_tokens, int64_t row_elems,
+                   int64_t key_stride, int64_t value_stride, int64_t n_slots,
+                   pdllm_stream_t stream);
+
+/* fp8 variant of the store (no reference counterpart beyond the scalar-scale
+ * branch of OPS/prefix_prefill.py:118-121): quantises bf16 rows to e4m3 with
+ * the scale of the destination page, x_q = e4m3(x / scale[page]).
+ * k_scale/v_scale: [n_pages] fp32, already filled by the caller. */
+int pdllm_kv_store_fp8(const void* key, const void* value, void* k_cache, void* v_cache,
+                       const float* k_scale, const float* v_scale,
+                       const int32_t* slot_mapping, int64_t n_tokens, int64_t row_elems,
+                       int64_t key_stride, int64_t value_stride, int64_t n_slots,
+                       int32_t page_size, pdllm_stream_t stream);
+
+/* Replaces the slot-mapping builders ENG:331-351, 434-441:
+ * slot[i] = page_ids[(start_token+i) / page_size] * page_size + (start_token+i) % page_size.
+ * page_ids: device int32 [n_page_ids]; tokens that fall beyond it get -1. */
+int pdllm_slot_mapping(const int32_t* page_ids, int64_t n_page_ids, int64_t start_token,
+                       int64_t n_tokens, int32_t page_size, int32_t* slots_out,
+                       pdllm_stream_t stream);
+
+/* Replaces load_kvcache + load_kvcache_kernel_kv (OPS/kv_cache_kernels.py:278-327,
+ * 175-275): per sequence s, k_out[cu_k[s] + t] = cache[block_table[s][t/P]][t%P]
+ * for t < ctx_len[s], followed by the sequence's active rows of k_new/v_new.
+ * 16-bit elements; all row strides in elements. */
+int pdllm_kv_load(const void* k_cache, const void* v_cache, const void* k_new, const void* v_new,
+                  void* k_out, void* v_out, const int32_t* block_table, int64_t bt_stride,
+                  const int32_t* ctx_lens, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                  int32_t n_seqs, int64_t max_total_len, int64_t row_elems, int32_t page_size,
+                  int64_t n_pages, int64_t new_stride, int64_t out_stride, pdllm_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Attention over non-contiguous chunk KV pages + the active block            *
+ * ------------------------------------------------------------------------- */
+
+typedef struct pdllm_attn_desc {
+  /* in-flight tensors, bf16, rows of head_dim contiguous elements */
+  const void* q;      /* [n_tokens, Hq, d]   token stride q_stride (elements)  */
+  const void* k_new;  /* [n_tokens, Hkv, d]  token stride kn_stride            */
+  const void* v_new;  /* [n_tokens, Hkv, d]  token stride vn_stride            */
+  void* out;          /* [n_tokens, Hq, d]   token stride o_stride             */
+  /* paged cache, unified layout [n_pages, page_size, Hkv, d]; NULL = no prefix */
+  const void* k_cache;
+  const void* v_cache;
+  const float* k_scale; /* fp8 only: scale[page*scale_page_stride + kvh*scale_head_stride] */
+  const float* v_scale;
+  const int32_t* block_table; /* [n_req, bt_stride] page ids (entries < 0 or >= n_pages read as zero rows) */
+  const int32_t* q_start_loc; /* [n_req+1] first active row of each request     */
+  /* visible prefix of request r = ranges range_ptr[r] .. range_ptr[r+1]-1, each a
+   * run of logical tokens [range_start, range_start+range_len) that is mapped
+   * through block_table[r][token / page_size]. */
+  const int32_t* range_ptr;   /* [n_req+1] */
+  const int32_t* range_start; /* [n_ranges] */
+  const int32_t* range_len;   /* [n_ranges] */
+  const uint8_t* mask; /* PDLLM_MASK_DENSE: bool[n_tokens, mask_stride], entry
+                          (q_start+i, q_start+j) = row i of the request sees active key j */
+  void* workspace;     /* split-KV partial results */
+  int64_t workspace_bytes;
+  int64_t q_stride, kn_stride, vn_stride, o_stride;           /* elements */
+  int64_t cache_page_stride, cache_token_stride, cache_head_stride; /* elements of the cache dtype */
+  int64_t mask_stride;
+  int64_t n_tokens; /* rows of q/k_new/v_new/out                              */
+  int64_t n_pages;
+  int32_t bt_stride;
+  int32_t scale_page_stride, scale_head_stride;
+  int32_t n_req;
+  int32_t max_q_len;   /* host upper bound of the per-request active length   */
+  int32_t max_ctx_len; /* host upper bound of the per-request visible prefix  */
+  int32_t max_ranges;  /* host upper bound of ranges per request (<= 128)     */
+  int32_t num_q_heads, num_kv_heads, head_dim; /* head_dim must be 128        */
+  int32_t page_size;   /* power of two                                        */
+  int32_t kv_dtype;    /* PDLLM_KV_*  (dtype of the cache; in-flight K/V are bf16) */
+  int32_t mask_mode;   /* PDLLM_MASK_*                                        */
+  int32_t num_splits;  /* 0 = choose; >0 = force this many KV splits          */
+  int32_t rows_per_group; /* 0 = choose; else 32*J, J in {1,2,4,5,6,8}        */
+  float sm_scale;      /* softmax scale (1/sqrt(d) when the caller has no own) */
+} pdllm_attn_desc;
+
+/* Bytes of workspace pdllm_sparse_decode_attn needs for this descriptor
+ * (0 when no KV split is used).  Negative = error code. */
+int64_t pdllm_attn_workspace_bytes(const pdllm_attn_desc* desc);
+
+/* Replaces the decode branch of Attention.forward (layers/attention/attention_v4.py:368-397),
+ * i.e. load_kvcache + flex/SDPA attention (unified layout) or
+ * diffusion_lm_parallel_flash_decoding = chunked_prefill_paged_decode ->
+ * context_attention_fwd -> _fwd_kernel_d2f (OPS/chunked_prefill_decoding_unified_kernel.py:220-274,
+ * OPS/prefix_prefill.py:25-230): out = softmax(Q K^T * sm_scale + mask) V over
+ * [selected prefix pages || active block], GQA by head grouping, fp32 softmax
+ * and accumulation.  Rows with no visible key produce zeros. */
+int pdllm_sparse_decode_attn(const pdllm_attn_desc* desc, pdllm_stream_t stream);
+
+/* Replaces the prefill branch of Attention.forward (attention_v4.py:336-367) for a
+ * packed batch of independent chunks (block-diagonal mask, context.py:73-84):
+ * per chunk c (rows cu_seqlens[c]..cu_seqlens[c+1]) causal or full
+ * self-attention, and (when slot_mapping != NULL) the paged store of K/V of
+ * OPS/kv_cache_kernels.py:150-172 for the same rows.  Uses the descriptor's
+ * in-flight tensors, q_start_loc (= cu_seqlens), mask_mode and cache fields. */
+int pdllm_chunk_prefill_attn(const pdllm_attn_desc* desc, const int32_t* slot_mapping,
+                             pdllm_stream_t stream);
+
+/* The plan pdllm_sparse_decode_attn (prefill == 0) or pdllm_chunk_prefill_attn would use:
+ * rows per workgroup (32 * row blocks) and number of KV splits.  For tuning and tests. */
+int pdllm_attn_plan(const pdllm_attn_desc* desc, int32_t prefill, int32_t* rows_per_group,
+                    int32_t* num_splits);
+
+/* ------------------------------------------------------------------------- *
+ * Chunk scoring and selection                                                *
+ * ------------------------------------------------------------------------- */
+
+/* Replaces F.log_softmax(...).gather(...) of score_chunk_self_information_engine
+ * (ENG:1148-1152) for a batch of rows: logp[r] = logits[r, label[r]] - logsumexp(logits[r,:])
+ * in fp32 over bf16 logits [n_rows, vocab] (row stride logits_stride elements).
+ * A label outside [0, vocab) yields -inf. */
+int pdllm_selfinfo_logprob(const void* logits, int64_t logits_stride, const int64_t* labels,
+                           int64_t n_rows, int64_t vocab, void* workspace, int64_t workspace_bytes,
+                           float* logp_out, pdllm_stream_t stream);
+
+/* Bytes of workspace the two vocabulary scans (pdllm_selfinfo_logprob, pdllm_conf_argmax)
+ * need for n_rows rows of `vocab` logits: per-row, per-split (max, sum, argmax) partials. */
+int64_t pdllm_vocab_workspace_bytes(int64_t n_rows, int64_t vocab);
+
+/* score[c] = (mean ? 1/rows_per_chunk : 1) * sum_j logp[c*rows_per_chunk + j], summed in
+ * index order in fp32 (ENG:1152 takes the mean). */
+int pdllm_chunk_score_reduce(const float* logp, int64_t n_chunks, int64_t rows_per_chunk,
+                             int32_t mean, float* scores_out, pdllm_stream_t stream);
+
+/* Replaces the ranking of select_chunks_by_engine (ENG:1199-1204): per row of
+ * scores [n_rows, n] (non-finite -> -inf), the k best indices by (score desc,
+ * index asc), returned ascending when sorted_ascending != 0, else in rank order.
+ * n <= 65536, k <= n. */
+int pdllm_topk_lowest_index(const float* scores, int64_t n_rows, int64_t n, int64_t scores_stride,
+                            int64_t k, int32_t sorted_ascending, int64_t* indices_out,
+                            pdllm_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Intra-chunk token eviction                                                 *
+ * ------------------------------------------------------------------------- */
+
+/* Column sums of ready-made attention probabilities: probs [n_chunks, n_heads,
+ * n_queries, n_keys] fp32 contiguous -> scores [n_chunks, n_groups, n_keys] with
+ * heads_per_group consecutive heads summed (n_groups = n_heads / heads_per_group;
+ * heads_per_group = n_heads gives the global score of
+ * prefilling_dllm_eval/fastdllm_parallelcomp.py:1607-1637).  The sum runs over
+ * (head, query) in index order, so it is reproducible bit for bit. */
+int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t n_heads, int64_t n_queries,
+                       int64_t n_keys, int64_t heads_per_group, float* scores_out,
+                       pdllm_stream_t stream);
+
+/* Replaces query_to_chunk_attention_scores (OPS/triton_eviction_scorer.py:114-210) and
+ * the torch path of _engine_chunk_attention_head_scores (ENG:1279-1310): q [S, Hq, d],
+ * k [S, Hkv, d] bf16 contiguous, S = prefix_len + chunk_len + query_len; for every
+ * q-head, softmax over the visible keys of the last query_len rows, summed (or averaged)
+ * over those rows on the chunk columns -> out [Hq, chunk_len] fp32.
+ * causal != 0: key j visible to row i iff j <= i.  workspace: 2*Hq*query_len floats. */
+int pdllm_evict_score_qk(const void* q, const void* k, int64_t prefix_len, int64_t chunk_len,
+                         int64_t query_len, int32_t num_q_heads, int32_t num_kv_heads,
+                         int32_t head_dim, float scale, int32_t reduce_mean, int32_t causal,
+                         float* workspace, float* out, pdllm_stream_t stream);
+
+/* Replaces the pooling + per-KV-head grouping of ENG:1405-1433: optional max/avg pool
+ * (kernel, padding kernel/2, stride 1, as F.max_pool1d / F.avg_pool1d with
+ * count_include_pad) over [n_heads, n] rows then the mean of each group of
+ * heads_per_group rows -> [n_heads/heads_per_group, n].  pool: 0 none, 1 max, 2 avg. */
+int pdllm_token_score_pool_group(const float* scores, int64_t n_heads, int64_t n, int32_t pool,
+                                 int32_t kernel, int64_t heads_per_group, float* out,
+                                 pdllm_stream_t stream);
+
+/* Replaces _select_positions_from_token_scores (ENG:903-927): per row of scores
+ * [n_rows, chunk_len]: keep position 0 (BOS) and the keep_count-1 best of positions
+ * 1..chunk_len-1 by (score desc, index asc); indices_out [n_rows, keep_count] ascending.
+ * keep_count = min(max(1, capacity), chunk_len).  keep_high == 0 ranks by (score asc,
+ * index asc).  force_keep_first == 0 ranks all positions. */
+int pdllm_topb_keep_bos(const float* scores, int64_t n_rows, int64_t chunk_len,
+                        int64_t scores_stride, int64_t capacity, int32_t keep_high,
+                        int32_t force_keep_first, int64_t* indices_out, pdllm_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * KV compaction / snapshot                                                   *
+ * ------------------------------------------------------------------------- */
+
+/* Replaces _snapshot_prompt_cache_per_layer / the gather half of
+ * _compact_prompt_cache_per_layer_per_head and _copy_chunk_local_kv_to_prompt_pages
+ * (ENG:640-662, 607-638, 525-558).  For token j < n_tokens and head h:
+ *   t = token_idx ? token_idx[h*idx_head_stride + j] + src_offset : j + src_offset
+ *   dst[j, h, :] = cache[page_ids[t / P], t % P, h, :]
+ * dst: dense [n_tokens, Hkv, d].  elem_bytes = bytes of one element (2 or 1). */
+int pdllm_kv_gather(const void* cache, const int32_t* page_ids, int64_t n_page_ids,
+                    const int64_t* token_idx, int64_t idx_head_stride, int64_t src_offset,
+                    int64_t n_tokens, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                    int64_t n_pages, int32_t elem_bytes, void* dst, pdllm_stream_t stream);
+
+/* Replaces _load_prompt_cache_per_layer / the scatter half of the functions above
+ * (ENG:664-698): cache[page_ids[(dst_start+j)/P], (dst_start+j)%P, h, :] = src[j, h, :]. */
+int pdllm_kv_scatter(void* cache, const int32_t* page_ids, int64_t n_page_ids, int64_t dst_start,
+                     int64_t n_tokens, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                     int64_t n_pages, int32_t elem_bytes, const void* src, pdllm_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Confidence-threshold unmasking                                             *
+ * ------------------------------------------------------------------------- */
+
+/* Replaces _shift_logits + _sample_tokens at temperature 0 (ENG:1647-1681) for
+ * n_seqs blocks of block_len rows of bf16 logits [n_seqs*block_len, vocab]:
+ * row i of block b reads logits row (b*block_len + i - shift) where shift = 1 uses
+ * last_logit[b] (or the block's own row 0 when last_logit == NULL) for i = 0;
+ * confidence = max softmax probability in fp32, token = first index of the maximum. */
+int pdllm_conf_argmax(const void* logits, int64_t logits_stride, const void* last_logit,
+                      int64_t last_logit_stride, int64_t n_seqs, int64_t block_len, int64_t vocab,
+                      int32_t shift, void* workspace, int64_t workspace_bytes, float* conf_out,
+                      int64_t* token_out, pdllm_stream_t stream);
+
+/* Replaces the transfer rule of decode_from_pd_record (ENG:2146-2157) without host
+ * syncs: per block b over the positions with block_ids == mask_token_id, transfer the
+ * most confident one (lowest index on ties) and every one with conf >= threshold;
+ * writes the tokens into block_ids in place, transfer_out[b, i] in {0,1} and
+ * n_masked_left[b] = masked positions remaining after the update. */
+int pdllm_threshold_unmask(const float* conf, const int64_t* token, int64_t* block_ids,
+                           int64_t n_seqs, int64_t block_len, int64_t mask_token_id,
+                           float threshold, uint8_t* transfer_out, int32_t* n_masked_left,
+                           pdllm_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Rotary embedding (the step in front of the path)                           *
+ * ------------------------------------------------------------------------- */
+
+/* Replaces RotaryEmbedding.forward / apply_rotary_emb (layers/rotary_embedding.py:6-17,
+ * 39-65): neox split-half rotation in fp32 with cos_sin_cache[positions] =
+ * [cos(d/2) | sin(d/2)] fp32 rows, applied in place to x [n_tokens, n_heads, d] bf16. */
+int pdllm_rope_inplace(void* x, int64_t x_stride, const int64_t* positions,
+                       const float* cos_sin_cache, int64_t max_positions, int64_t n_tokens,
+                       int32_t n_heads, int32_t head_dim, pdllm_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PDLLM_H */

@@ -1,0 +1,343 @@
+// Vocabulary-wide reductions over bf16 logits for gfx950: draft self-information
+// (log-softmax of a label), max-softmax confidence + argmax, and the threshold unmask rule.
+// These are single-pass HBM-bound scans: every lane streams 16-byte (8 x bf16) loads, keeps a
+// lane-local online (max, sum-of-exp[, argmax]) and the lanes are combined with wavefront
+// reductions.  A row is split over several workgroups so that a few hundred rows still fill
+// 256 CUs; the per-split partials are combined by a second tiny kernel in split order.
+//
+// Reference: fastdllm_engine.py:1148-1152 (self-information), :1647-1681 (shift + confidence),
+// :2146-2157 (transfer rule) of the reference engine.
+
+#include "pdllm_common.h"
+
+namespace pdllm {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct RowStat {
+  float m;   // running maximum
+  float s;   // sum of exp(x - m)
+  long idx;  // first index of the maximum
+};
+
+__device__ __forceinline__ void stat_merge(RowStat& a, const RowStat& b) {
+  // maximum with lowest-index tie-break, sums rescaled to the common maximum
+  const bool b_wins = (b.m > a.m) || (b.m == a.m && b.idx < a.idx);
+  const float mm = fmaxf(a.m, b.m);
+  const float sa = (a.m == -INFINITY) ? 0.f : a.s * __builtin_amdgcn_exp2f((a.m - mm) * kLog2e);
+  const float sb = (b.m == -INFINITY) ? 0.f : b.s * __builtin_amdgcn_exp2f((b.m - mm) * kLog2e);
+  a.s = sa + sb;
+  a.m = mm;
+  if (b_wins) a.idx = b.idx;
+}
+
+__device__ __forceinline__ void stat_push(RowStat& st, float x, long i) {
+  if (x > st.m) {
+    st.s = st.s * __builtin_amdgcn_exp2f((st.m - x) * kLog2e) + 1.f;  // st.m = -inf -> 0
+    st.m = x;
+    st.idx = i;
+  } else {
+    st.s += __builtin_amdgcn_exp2f((x - st.m) * kLog2e);
+  }
+}
+
+// partial[(row * nsplit + split)] = stats of logits[row, split segment]
+__global__ __launch_bounds__(256) void vocab_partial_kernel(
+    const __bf16* __restrict__ logits, long logits_stride, const __bf16* __restrict__ last_logit,
+    long last_stride, long block_len, int shift, long vocab, int nsplit, float* __restrict__ part_m,
+    float* __restrict__ part_s, long* __restrict__ part_idx) {
+  const long row = blockIdx.y;
+  const int split = blockIdx.x;
+  // source row after the optional one-position shift inside each block
+  const __bf16* src;
+  if (shift) {
+    const long b = row / block_len, i = row - b * block_len;
+    if (i == 0) src = last_logit ? last_logit + b * last_stride : logits + row * logits_stride;
+    else src = logits + (row - 1) * logits_stride;
+  } else {
+    src = logits + row * logits_stride;
+  }
+  const long seg = (((vocab + nsplit - 1) / nsplit) + 7) & ~7L;  // multiple of 8 elements
+  const long begin = (long)split * seg;
+  long end = begin + seg;
+  end = end < vocab ? end : vocab;
+
+  RowStat st = {-INFINITY, 0.f, 0x7fffffffffffffffL};
+  const bool vec_ok = (((uintptr_t)src) % 16) == 0;
+  if (vec_ok) {
+    for (long i = begin + 8L * threadIdx.x; i < end; i += 8L * 256) {
+      if (i + 8 <= end) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(src + i);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+        float x[8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          x[2 * k] = bf16_bits_to_f32(w[k] & 0xffffu);
+          x[2 * k + 1] = bf16_bits_to_f32(w[k] >> 16);
+        }
+        // vector step: one rescale for the 8 values
+        float vm = x[0];
+        int vi = 0;
+#pragma unroll
+        for (int k = 1; k < 8; ++k)
+          if (x[k] > vm) { vm = x[k]; vi = k; }
+        if (vm > st.m) {
+          st.s *= __builtin_amdgcn_exp2f((st.m - vm) * kLog2e);
+          st.m = vm;
+          st.idx = i + vi;
+        }
+        if (st.m > -INFINITY) {
+          float acc = 0.f;
+#pragma unroll
+          for (int k = 0; k < 8; ++k) acc += __builtin_amdgcn_exp2f((x[k] - st.m) * kLog2e);
+          st.s += acc;
+        }
+      } else {
+        for (long j = i; j < end; ++j)
+          stat_push(st, bf16_bits_to_f32(__builtin_bit_cast(unsigned short, src[j])), j);
+      }
+    }
+  } else {
+    for (long j = begin + threadIdx.x; j < end; j += 256)
+      stat_push(st, bf16_bits_to_f32(__builtin_bit_cast(unsigned short, src[j])), j);
+  }
+  // wave reduction, then across the 4 waves through LDS
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    RowStat other;
+    other.m = __shfl_xor(st.m, o, 64);
+    other.s = __shfl_xor(st.s, o, 64);
+    other.idx = __shfl_xor(st.idx, o, 64);
+    stat_merge(st, other);
+  }
+  __shared__ float sm[4], ss[4];
+  __shared__ long si[4];
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) { sm[wave] = st.m; ss[wave] = st.s; si[wave] = st.idx; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    RowStat a = {sm[0], ss[0], si[0]};
+    for (int w = 1; w < 4; ++w) {
+      RowStat b = {sm[w], ss[w], si[w]};
+      stat_merge(a, b);
+    }
+    const long o = row * nsplit + split;
+    part_m[o] = a.m;
+    part_s[o] = a.s;
+    part_idx[o] = a.idx;
+  }
+}
+
+// mode 0: logp[row] = logits[row, label] - logsumexp ; mode 1: conf = 1 / sum exp(x - max), token = argmax
+__global__ __launch_bounds__(64) void vocab_final_kernel(
+    const float* __restrict__ part_m, const float* __restrict__ part_s, const long* __restrict__ part_idx,
+    int nsplit, long n_rows, int mode, const __bf16* __restrict__ logits, long logits_stride,
+    const long* __restrict__ labels, long vocab, float* __restrict__ out_f, long* __restrict__ out_i) {
+  const long row = (long)blockIdx.x * 64 + threadIdx.x;
+  if (row >= n_rows) return;
+  RowStat a = {part_m[row * nsplit], part_s[row * nsplit], part_idx[row * nsplit]};
+  for (int s = 1; s < nsplit; ++s) {
+    RowStat b = {part_m[row * nsplit + s], part_s[row * nsplit + s], part_idx[row * nsplit + s]};
+    stat_merge(a, b);
+  }
+  if (mode == 0) {
+    const long lab = labels[row];
+    float r = -INFINITY;
+    if (lab >= 0 && lab < vocab) {
+      const float x = bf16_bits_to_f32(__builtin_bit_cast(unsigned short, logits[row * logits_stride + lab]));
+      r = (x - a.m) - __log2f(a.s) * kLn2;
+    }
+    out_f[row] = r;
+  } else {
+    out_f[row] = 1.f / a.s;
+    out_i[row] = a.idx;
+  }
+}
+
+__global__ __launch_bounds__(64) void chunk_score_reduce_kernel(const float* __restrict__ logp,
+                                                                long n_chunks, long rows_per_chunk,
+                                                                int mean, float* __restrict__ out) {
+  const long c = (long)blockIdx.x * 64 + threadIdx.x;
+  if (c >= n_chunks) return;
+  float acc = 0.f;
+  for (long j = 0; j < rows_per_chunk; ++j) acc += logp[c * rows_per_chunk + j];
+  out[c] = mean ? acc / (float)rows_per_chunk : acc;
+}
+
+// one wave per block of the batch
+__global__ __launch_bounds__(64) void threshold_unmask_kernel(
+    const float* __restrict__ conf, const long* __restrict__ token, long* __restrict__ block_ids,
+    long block_len, long mask_token_id, float threshold, uint8_t* __restrict__ transfer,
+    int* __restrict__ n_left) {
+  const long b = blockIdx.x;
+  const int lane = threadIdx.x;
+  const long base = b * block_len;
+  // pass 1: most confident masked position (lowest index on ties)
+  float best = -INFINITY;
+  long besti = 0x7fffffffffffffffL;
+  int n_masked = 0;
+  for (long i = lane; i < block_len; i += 64) {
+    if (block_ids[base + i] == mask_token_id) {
+      ++n_masked;
+      const float c = conf[base + i];
+      if (c > best || besti == 0x7fffffffffffffffL) { best = c; besti = i; }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const long oi = __shfl_xor(besti, o, 64);
+    n_masked += __shfl_xor(n_masked, o, 64);
+    const bool o_valid = oi != 0x7fffffffffffffffL, s_valid = besti != 0x7fffffffffffffffL;
+    const bool take = o_valid && (!s_valid || ob > best || (ob == best && oi < besti));
+    if (take) { best = ob; besti = oi; }
+  }
+  int moved = 0;
+  for (long i = lane; i < block_len; i += 64) {
+    const bool masked = block_ids[base + i] == mask_token_id;
+    const bool t = masked && (i == besti || conf[base + i] >= threshold);
+    transfer[base + i] = t ? 1 : 0;
+    if (t) { block_ids[base + i] = token[base + i]; ++moved; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) moved += __shfl_xor(moved, o, 64);
+  if (lane == 0 && n_left) n_left[b] = n_masked - moved;
+}
+
+// neox rotary embedding in place: x [n_tokens, n_heads, d] bf16
+__global__ __launch_bounds__(256) void rope_kernel(__bf16* __restrict__ x, long x_stride,
+                                                   const long* __restrict__ positions,
+                                                   const float* __restrict__ cos_sin, long max_pos,
+                                                   long n_tokens, int n_heads, int head_dim) {
+  const int half = head_dim / 2;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const long per_tok = (long)n_heads * half;
+  const long t = idx / per_tok;
+  if (t >= n_tokens) return;
+  const int rem = (int)(idx - t * per_tok);
+  const int hd = rem / half, i = rem - hd * half;
+  const long pos = positions[t];
+  if (pos < 0 || pos >= max_pos) return;
+  const float c = cos_sin[pos * head_dim + i];
+  const float s = cos_sin[pos * head_dim + half + i];
+  __bf16* p = x + t * x_stride + (long)hd * head_dim;
+  const float x1 = (float)p[i], x2 = (float)p[i + half];
+  // fp32 products rounded separately, as the unfused torch expression
+  const float y1 = __fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s));
+  const float y2 = __fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, s));
+  p[i] = (__bf16)y1;
+  p[i + half] = (__bf16)y2;
+}
+
+static int vocab_nsplit(long n_rows, long vocab) {
+  // aim at >= 1024 workgroups, at least 2048 elements per workgroup
+  long want = (1024 + n_rows - 1) / n_rows;
+  const long max_by_len = (vocab + 2047) / 2048;
+  if (want > max_by_len) want = max_by_len;
+  if (want < 1) want = 1;
+  if (want > 64) want = 64;
+  return (int)want;
+}
+
+static int64_t vocab_ws_bytes(long n_rows, long vocab) {
+  const int ns = vocab_nsplit(n_rows, vocab);
+  return (int64_t)n_rows * ns * (4 + 4 + 8);
+}
+
+static int vocab_launch(const void* logits, int64_t logits_stride, const void* last_logit,
+                        int64_t last_stride, int64_t n_rows, int64_t block_len, int64_t vocab, int shift,
+                        int mode, const int64_t* labels, void* workspace, int64_t workspace_bytes,
+                        float* out_f, int64_t* out_i, hipStream_t stream) {
+  if (!logits || !out_f || !workspace) return PDLLM_ERR_NULL;
+  if (mode == 0 && !labels) return PDLLM_ERR_NULL;
+  if (mode == 1 && !out_i) return PDLLM_ERR_NULL;
+  if (n_rows < 0 || vocab <= 0 || logits_stride < vocab || block_len <= 0) return PDLLM_ERR_SHAPE;
+  if (n_rows > 65535) return PDLLM_ERR_UNSUPPORTED;
+  if (n_rows == 0) return PDLLM_OK;
+  if (workspace_bytes < vocab_ws_bytes(n_rows, vocab) || ((uintptr_t)workspace % 8)) return PDLLM_ERR_WORKSPACE;
+  const int ns = vocab_nsplit(n_rows, vocab);
+  long* pi = static_cast<long*>(workspace);
+  float* pm = reinterpret_cast<float*>(pi + n_rows * ns);
+  float* ps = pm + n_rows * ns;
+  hipLaunchKernelGGL(vocab_partial_kernel, dim3((unsigned)ns, (unsigned)n_rows), dim3(256), 0, stream,
+                     static_cast<const __bf16*>(logits), (long)logits_stride,
+                     static_cast<const __bf16*>(last_logit), (long)last_stride, (long)block_len, shift,
+                     (long)vocab, ns, pm, ps, pi);
+  int st = launch_status();
+  if (st != PDLLM_OK) return st;
+  hipLaunchKernelGGL(vocab_final_kernel, dim3((unsigned)((n_rows + 63) / 64)), dim3(64), 0, stream, pm, ps,
+                     pi, ns, (long)n_rows, mode, static_cast<const __bf16*>(logits), (long)logits_stride,
+                     reinterpret_cast<const long*>(labels), (long)vocab, out_f,
+                     reinterpret_cast<long*>(out_i));
+  return launch_status();
+}
+
+}  // namespace pdllm
+
+using namespace pdllm;
+
+extern "C" int64_t pdllm_vocab_workspace_bytes(int64_t n_rows, int64_t vocab) {
+  if (n_rows < 0 || vocab <= 0) return PDLLM_ERR_SHAPE;
+  if (n_rows == 0) return 0;
+  return vocab_ws_bytes(n_rows, vocab);
+}
+
+extern "C" int pdllm_selfinfo_logprob(const void* logits, int64_t logits_stride, const int64_t* labels,
+                                      int64_t n_rows, int64_t vocab, void* workspace,
+                                      int64_t workspace_bytes, float* logp_out, pdllm_stream_t stream) {
+  return vocab_launch(logits, logits_stride, nullptr, 0, n_rows, 1, vocab, 0, 0, labels, workspace,
+                      workspace_bytes, logp_out, nullptr, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pdllm_chunk_score_reduce(const float* logp, int64_t n_chunks, int64_t rows_per_chunk,
+                                        int32_t mean, float* scores_out, pdllm_stream_t stream) {
+  if (!logp || !scores_out) return PDLLM_ERR_NULL;
+  if (n_chunks < 0 || rows_per_chunk <= 0) return PDLLM_ERR_SHAPE;
+  if (n_chunks == 0) return PDLLM_OK;
+  hipLaunchKernelGGL(chunk_score_reduce_kernel, dim3((unsigned)((n_chunks + 63) / 64)), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), logp, (long)n_chunks, (long)rows_per_chunk, mean,
+                     scores_out);
+  return launch_status();
+}
+
+extern "C" int pdllm_conf_argmax(const void* logits, int64_t logits_stride, const void* last_logit,
+                                 int64_t last_logit_stride, int64_t n_seqs, int64_t block_len,
+                                 int64_t vocab, int32_t shift, void* workspace, int64_t workspace_bytes,
+                                 float* conf_out, int64_t* token_out, pdllm_stream_t stream) {
+  if (n_seqs < 0 || block_len <= 0) return PDLLM_ERR_SHAPE;
+  if (last_logit && last_logit_stride < vocab) return PDLLM_ERR_STRIDE;
+  return vocab_launch(logits, logits_stride, last_logit, last_logit_stride, n_seqs * block_len, block_len,
+                      vocab, shift ? 1 : 0, 1, nullptr, workspace, workspace_bytes, conf_out, token_out,
+                      static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pdllm_threshold_unmask(const float* conf, const int64_t* token, int64_t* block_ids,
+                                      int64_t n_seqs, int64_t block_len, int64_t mask_token_id,
+                                      float threshold, uint8_t* transfer_out, int32_t* n_masked_left,
+                                      pdllm_stream_t stream) {
+  if (!conf || !token || !block_ids || !transfer_out) return PDLLM_ERR_NULL;
+  if (n_seqs < 0 || block_len <= 0) return PDLLM_ERR_SHAPE;
+  if (n_seqs == 0) return PDLLM_OK;
+  if (n_seqs > 0x7fffffffL) return PDLLM_ERR_SHAPE;
+  hipLaunchKernelGGL(threshold_unmask_kernel, dim3((unsigned)n_seqs), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), conf, reinterpret_cast<const long*>(token),
+                     reinterpret_cast<long*>(block_ids), (long)block_len, (long)mask_token_id, threshold,
+                     transfer_out, n_masked_left);
+  return launch_status();
+}
+
+extern "C" int pdllm_rope_inplace(void* x, int64_t x_stride, const int64_t* positions,
+                                  const float* cos_sin_cache, int64_t max_positions, int64_t n_tokens,
+                                  int32_t n_heads, int32_t head_dim, pdllm_stream_t stream) {
+  if (!x || !positions || !cos_sin_cache) return PDLLM_ERR_NULL;
+  if (n_tokens < 0 || n_heads <= 0 || head_dim <= 0 || (head_dim & 1) || max_positions <= 0) return PDLLM_ERR_SHAPE;
+  if (x_stride < (int64_t)n_heads * head_dim) return PDLLM_ERR_STRIDE;
+  if (n_tokens == 0) return PDLLM_OK;
+  const long total = n_tokens * n_heads * (head_dim / 2);
+  hipLaunchKernelGGL(rope_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<__bf16*>(x), (long)x_stride,
+                     reinterpret_cast<const long*>(positions), cos_sin_cache, (long)max_positions,
+                     (long)n_tokens, n_heads, head_dim);
+  return launch_status();
+}

@@ -1,0 +1,428 @@
+// Selection kernels for gfx950: top-K of chunk scores, BOS-forced top-B of token scores
+// (both with a total order: score first, lowest index on ties), column sums of attention
+// probabilities, the query-to-chunk eviction scorer and token-score pooling.
+//
+// Reference: fastdllm_engine.py:1199-1204 (chunk ranking), :903-927 (token keep set),
+// :1230-1322 + layers/attention/ops/triton_eviction_scorer.py:6-210 (eviction scores),
+// :1405-1433 (pooling and per-KV-head grouping) of the reference engine.
+
+#include "pdllm_common.h"
+
+namespace pdllm {
+
+// Monotone map float -> uint32: a < b  <=>  ord(a) < ord(b); NaN above +inf.
+__device__ __forceinline__ uint32_t float_ord(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;  // NaN: largest
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// 64-bit sort key, smaller = better.  descending: high score first.
+__device__ __forceinline__ uint64_t make_key(float score, uint32_t idx, bool descending) {
+  const uint32_t o = float_ord(score);
+  const uint32_t hi = descending ? ~o : o;
+  return ((uint64_t)hi << 32) | idx;
+}
+
+constexpr int kSortMax = 2048;
+
+// in-LDS bitonic sort (ascending) of npad (power of two <= kSortMax) keys by 256 threads
+__device__ void bitonic_sort(uint64_t* keys, int npad) {
+  for (int k = 2; k <= npad; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int i = threadIdx.x; i < npad; i += 256) {
+        const int ixj = i ^ j;
+        if (ixj > i) {
+          const uint64_t a = keys[i], b = keys[ixj];
+          const bool up = (i & k) == 0;
+          if ((a > b) == up) { keys[i] = b; keys[ixj] = a; }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// One workgroup per row, n <= kSortMax.
+// mode 0: plain top-k (non-finite scores rank as -inf), mode 1: position 0 forced first.
+__global__ __launch_bounds__(256) void topk_sort_kernel(const float* __restrict__ scores, long n,
+                                                        long stride, long k, int descending,
+                                                        int force_first, int nonfinite_to_neginf,
+                                                        int sorted_ascending, long* __restrict__ out) {
+  __shared__ uint64_t keys[kSortMax];
+  __shared__ int flags[kSortMax];
+  __shared__ int wave_tot[4];
+  const long row = blockIdx.x;
+  const float* s = scores + row * stride;
+  int npad = 1;
+  while (npad < n) npad <<= 1;
+  for (int i = threadIdx.x; i < npad; i += 256) {
+    uint64_t key = ~0ull;  // padding sorts last
+    if (i < n) {
+      float v = s[i];
+      if (nonfinite_to_neginf && !(fabsf(v) <= 3.402823466e38f)) v = -INFINITY;
+      key = make_key(v, (uint32_t)i, descending != 0);
+      if (force_first && i == 0) key = 0ull;
+    }
+    keys[i] = key;
+    flags[i] = 0;
+  }
+  __syncthreads();
+  bitonic_sort(keys, npad);
+  if (!sorted_ascending) {
+    for (int i = threadIdx.x; i < k; i += 256) out[row * k + i] = (long)(keys[i] & 0xffffffffu);
+    return;
+  }
+  for (int i = threadIdx.x; i < k; i += 256) flags[(int)(keys[i] & 0xffffffffu)] = 1;
+  __syncthreads();
+  // ordered compaction of the flagged indices: each thread owns a contiguous span
+  const int span = npad / 256 > 0 ? npad / 256 : 1;
+  const int begin = threadIdx.x * span;
+  int cnt = 0;
+  for (int i = begin; i < begin + span && i < npad; ++i) cnt += flags[i];
+  // exclusive scan of cnt over the workgroup
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = cnt;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int v = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += v;
+  }
+  if (lane == 63) wave_tot[wave] = incl;
+  __syncthreads();
+  int base = incl - cnt;
+  for (int w = 0; w < wave; ++w) base += wave_tot[w];
+  for (int i = begin; i < begin + span && i < npad; ++i)
+    if (flags[i]) out[row * k + base++] = i;
+}
+
+// Radix select for long rows (n up to 65536): finds the k-th best 32-bit key, then keeps all
+// better keys and the lowest-index ties.  Output ascending by index.  One workgroup per row.
+__global__ __launch_bounds__(256) void topk_radix_kernel(const float* __restrict__ scores, long n,
+                                                         long stride, long k, int descending,
+                                                         int force_first, int nonfinite_to_neginf,
+                                                         long* __restrict__ out) {
+  __shared__ int hist[256];
+  __shared__ uint32_t s_prefix;
+  __shared__ int s_need;
+  __shared__ int wave_tot[4][2];
+  const long row = blockIdx.x;
+  const float* s = scores + row * stride;
+  auto key_of = [&](long i) -> uint32_t {
+    float v = s[i];
+    if (nonfinite_to_neginf && !(fabsf(v) <= 3.402823466e38f)) v = -INFINITY;
+    const uint32_t o = float_ord(v);
+    uint32_t kk = descending ? ~o : o;  // smaller = better
+    if (force_first && i == 0) kk = 0u;
+    return kk;
+  };
+  // note: with force_first the forced element shares key 0 only with scores that map to 0,
+  // i.e. +NaN in descending order; index order still puts position 0 first.
+  if (threadIdx.x == 0) { s_prefix = 0u; s_need = (int)k; }
+  __syncthreads();
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    hist[threadIdx.x] = 0;
+    __syncthreads();
+    const uint32_t prefix = s_prefix;
+    const uint32_t pmask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
+    for (long i = threadIdx.x; i < n; i += 256) {
+      const uint32_t kk = key_of(i);
+      if ((kk & pmask) == prefix) atomicAdd(&hist[(kk >> shift) & 255], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int need = s_need, b = 0;
+      for (; b < 256; ++b) {
+        if (hist[b] >= need) break;
+        need -= hist[b];
+      }
+      s_need = need;
+      s_prefix = prefix | ((uint32_t)b << shift);
+    }
+    __syncthreads();
+  }
+  const uint32_t kth = s_prefix;  // key of the k-th best element
+  const int need_eq = s_need;     // how many elements equal to kth are kept (lowest indices)
+  // ordered compaction: thread owns a contiguous span of indices
+  const long span = (n + 255) / 256;
+  const long begin = threadIdx.x * span;
+  long end = begin + span;
+  end = end < n ? end : n;
+  int c_lt = 0, c_eq = 0;
+  for (long i = begin; i < end; ++i) {
+    const uint32_t kk = key_of(i);
+    c_lt += kk < kth;
+    c_eq += kk == kth;
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int i_lt = c_lt, i_eq = c_eq;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int a = __shfl_up(i_lt, o, 64), b = __shfl_up(i_eq, o, 64);
+    if (lane >= o) { i_lt += a; i_eq += b; }
+  }
+  if (lane == 63) { wave_tot[wave][0] = i_lt; wave_tot[wave][1] = i_eq; }
+  __syncthreads();
+  int b_lt = i_lt - c_lt, b_eq = i_eq - c_eq;
+  for (int w = 0; w < wave; ++w) { b_lt += wave_tot[w][0]; b_eq += wave_tot[w][1]; }
+  // position in the output = (#kept with lower index)
+  for (long i = begin; i < end; ++i) {
+    const uint32_t kk = key_of(i);
+    const int eq_kept_before = b_eq < need_eq ? b_eq : need_eq;
+    if (kk < kth) {
+      out[row * k + b_lt + eq_kept_before] = i;
+      ++b_lt;
+    } else if (kk == kth) {
+      if (b_eq < need_eq) out[row * k + b_lt + b_eq] = i;
+      ++b_eq;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// column sums of probabilities: out[c, g, k] = sum_{h in group g} ( sum_q p[c, h, q, k] )
+// inner sums run over q in index order, then heads in index order (fixed, reproducible).
+// ---------------------------------------------------------------------------------------
+constexpr int kColBlock = 64;
+
+__global__ __launch_bounds__(256) void evict_colsum_kernel(const float* __restrict__ probs, long n_heads,
+                                                           long n_q, long n_keys, long hpg,
+                                                           float* __restrict__ out) {
+  extern __shared__ float head_sum[];  // [n_heads][kColBlock]
+  const long chunk = blockIdx.y;
+  const long col = (long)blockIdx.x * kColBlock + (threadIdx.x & 63);
+  const int sub = threadIdx.x >> 6;
+  const float* base = probs + chunk * n_heads * n_q * n_keys;
+  for (long hd = sub; hd < n_heads; hd += 4) {
+    float acc = 0.f;
+    if (col < n_keys) {
+      const float* p = base + hd * n_q * n_keys + col;
+      long q = 0;
+      for (; q + 8 <= n_q; q += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p[(q + u) * n_keys];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += v[u];
+      }
+      for (; q < n_q; ++q) acc += p[q * n_keys];
+    }
+    head_sum[hd * kColBlock + (threadIdx.x & 63)] = acc;
+  }
+  __syncthreads();
+  const long n_groups = n_heads / hpg;
+  for (long g = sub; g < n_groups; g += 4) {
+    float acc = 0.f;
+    for (long hh = 0; hh < hpg; ++hh) acc += head_sum[(g * hpg + hh) * kColBlock + (threadIdx.x & 63)];
+    if (col < n_keys) out[(chunk * n_groups + g) * n_keys + col] = acc;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// query-to-chunk eviction scorer from q / k (bf16), fp32 math
+// ---------------------------------------------------------------------------------------
+// pass 1: one workgroup per (q-head, query row): softmax max and denominator over visible keys
+__global__ __launch_bounds__(256) void evict_maxden_kernel(const __bf16* __restrict__ q,
+                                                           const __bf16* __restrict__ k, long prefix_len,
+                                                           long chunk_len, long query_len, int Hq, int Hkv,
+                                                           int d, float scale, int causal,
+                                                           float* __restrict__ mx, float* __restrict__ den) {
+  __shared__ float qrow[256];
+  __shared__ float red_m[4], red_s[4];
+  const int head = blockIdx.x, qi = blockIdx.y;
+  const int kvh = head / (Hq / Hkv);
+  const long row = prefix_len + chunk_len + qi;
+  const long key_len = prefix_len + chunk_len + query_len;
+  for (int i = threadIdx.x; i < d; i += 256) qrow[i] = (float)q[(row * Hq + head) * d + i];
+  __syncthreads();
+  const long last = causal ? row : key_len - 1;
+  float m = -INFINITY, s = 0.f;
+  for (long j = threadIdx.x; j <= last; j += 256) {
+    const __bf16* kp = k + (j * Hkv + kvh) * d;
+    float acc = 0.f;
+    for (int i = 0; i < d; ++i) acc += (float)kp[i] * qrow[i];
+    const float x = acc * scale;
+    if (x > m) { s = s * __expf(m - x) + 1.f; m = x; }
+    else s += __expf(x - m);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float om = __shfl_xor(m, o, 64), os = __shfl_xor(s, o, 64);
+    const float mm = fmaxf(m, om);
+    s = (m == -INFINITY ? 0.f : s * __expf(m - mm)) + (om == -INFINITY ? 0.f : os * __expf(om - mm));
+    m = mm;
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) { red_m[wave] = m; red_s[wave] = s; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float M = red_m[0], S = red_s[0];
+    for (int w = 1; w < 4; ++w) {
+      const float mm = fmaxf(M, red_m[w]);
+      S = (M == -INFINITY ? 0.f : S * __expf(M - mm)) + (red_m[w] == -INFINITY ? 0.f : red_s[w] * __expf(red_m[w] - mm));
+      M = mm;
+    }
+    mx[head * query_len + qi] = M;
+    den[head * query_len + qi] = S;
+  }
+}
+
+// pass 2: one thread per (q-head, chunk column): sum over the query rows in index order
+__global__ __launch_bounds__(64) void evict_chunk_scores_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ k, const float* __restrict__ mx,
+    const float* __restrict__ den, long prefix_len, long chunk_len, long query_len, int Hq, int Hkv, int d,
+    float scale, int reduce_mean, float* __restrict__ out) {
+  extern __shared__ float qs[];  // [query_len][d]
+  const int head = blockIdx.x;
+  const int kvh = head / (Hq / Hkv);
+  const long c = (long)blockIdx.y * 64 + threadIdx.x;
+  const long qrow0 = prefix_len + chunk_len;
+  for (long i = threadIdx.x; i < query_len * d; i += 64) {
+    const long qi = i / d, e = i - qi * d;
+    qs[i] = (float)q[((qrow0 + qi) * Hq + head) * d + e];
+  }
+  __syncthreads();
+  if (c >= chunk_len) return;
+  const __bf16* kp = k + ((prefix_len + c) * Hkv + kvh) * d;
+  float acc = 0.f;
+  for (long qi = 0; qi < query_len; ++qi) {
+    float dot = 0.f;
+    for (int e = 0; e < d; ++e) dot += (float)kp[e] * qs[qi * d + e];
+    // chunk columns precede every query row, so they are visible under a causal mask too
+    acc += __expf(dot * scale - mx[head * query_len + qi]) / den[head * query_len + qi];
+  }
+  out[(long)head * chunk_len + c] = reduce_mean ? acc / (float)query_len : acc;
+}
+
+// pooling (max / avg, stride 1, padding kernel/2) then mean over groups of heads
+__global__ __launch_bounds__(256) void pool_group_kernel(const float* __restrict__ scores, long n_heads,
+                                                         long n, int pool, int kernel, long hpg,
+                                                         float* __restrict__ out) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  const long g = blockIdx.y;
+  if (i >= n) return;
+  const int pad = kernel / 2;
+  float acc = 0.f;
+  for (long hh = 0; hh < hpg; ++hh) {
+    const float* s = scores + (g * hpg + hh) * n;
+    float v;
+    if (pool == 0) {
+      v = s[i];
+    } else if (pool == 1) {
+      v = -INFINITY;
+      for (int w = 0; w < kernel; ++w) {
+        const long j = i - pad + w;
+        if (j >= 0 && j < n) v = fmaxf(v, s[j]);
+      }
+    } else {
+      float t = 0.f;
+      for (int w = 0; w < kernel; ++w) {
+        const long j = i - pad + w;
+        if (j >= 0 && j < n) t += s[j];
+      }
+      v = t / (float)kernel;
+    }
+    acc += v;
+  }
+  out[g * n + i] = hpg > 1 ? acc / (float)hpg : acc;
+}
+
+static int topk_launch(const float* scores, int64_t n_rows, int64_t n, int64_t stride, int64_t k,
+                       int descending, int force_first, int nonfinite, int sorted_ascending,
+                       int64_t* out, hipStream_t stream) {
+  if (!scores || !out) return PDLLM_ERR_NULL;
+  if (n_rows < 0 || n <= 0 || k < 0 || k > n || stride < n || n > 65536) return PDLLM_ERR_SHAPE;
+  if (n_rows == 0 || k == 0) return PDLLM_OK;
+  if (n_rows > 0x7fffffffL) return PDLLM_ERR_SHAPE;
+  if (n <= kSortMax) {
+    hipLaunchKernelGGL(topk_sort_kernel, dim3((unsigned)n_rows), dim3(256), 0, stream, scores, (long)n,
+                       (long)stride, (long)k, descending, force_first, nonfinite, sorted_ascending,
+                       reinterpret_cast<long*>(out));
+  } else {
+    if (!sorted_ascending) return PDLLM_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(topk_radix_kernel, dim3((unsigned)n_rows), dim3(256), 0, stream, scores, (long)n,
+                       (long)stride, (long)k, descending, force_first, nonfinite,
+                       reinterpret_cast<long*>(out));
+  }
+  return launch_status();
+}
+
+}  // namespace pdllm
+
+using namespace pdllm;
+
+extern "C" int pdllm_topk_lowest_index(const float* scores, int64_t n_rows, int64_t n,
+                                       int64_t scores_stride, int64_t k, int32_t sorted_ascending,
+                                       int64_t* indices_out, pdllm_stream_t stream) {
+  return topk_launch(scores, n_rows, n, scores_stride, k, 1, 0, 1, sorted_ascending, indices_out,
+                     static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pdllm_topb_keep_bos(const float* scores, int64_t n_rows, int64_t chunk_len,
+                                   int64_t scores_stride, int64_t capacity, int32_t keep_high,
+                                   int32_t force_keep_first, int64_t* indices_out,
+                                   pdllm_stream_t stream) {
+  if (chunk_len <= 0) return PDLLM_ERR_SHAPE;
+  int64_t keep = capacity < 1 ? 1 : capacity;
+  if (keep > chunk_len) keep = chunk_len;
+  return topk_launch(scores, n_rows, chunk_len, scores_stride, keep, keep_high ? 1 : 0,
+                     force_keep_first ? 1 : 0, 0, 1, indices_out, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t n_heads,
+                                  int64_t n_queries, int64_t n_keys, int64_t heads_per_group,
+                                  float* scores_out, pdllm_stream_t stream) {
+  if (!probs || !scores_out) return PDLLM_ERR_NULL;
+  if (n_chunks < 0 || n_heads <= 0 || n_queries <= 0 || n_keys <= 0 || heads_per_group <= 0 ||
+      n_heads % heads_per_group)
+    return PDLLM_ERR_SHAPE;
+  if (n_chunks == 0) return PDLLM_OK;
+  if (n_chunks > 65535 || n_heads * kColBlock * 4 > 64 * 1024) return PDLLM_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)((n_keys + kColBlock - 1) / kColBlock), (unsigned)n_chunks);
+  hipLaunchKernelGGL(evict_colsum_kernel, grid, dim3(256), (size_t)(n_heads * kColBlock * 4),
+                     static_cast<hipStream_t>(stream), probs, (long)n_heads, (long)n_queries, (long)n_keys,
+                     (long)heads_per_group, scores_out);
+  return launch_status();
+}
+
+extern "C" int pdllm_evict_score_qk(const void* q, const void* k, int64_t prefix_len, int64_t chunk_len,
+                                    int64_t query_len, int32_t num_q_heads, int32_t num_kv_heads,
+                                    int32_t head_dim, float scale, int32_t reduce_mean, int32_t causal,
+                                    float* workspace, float* out, pdllm_stream_t stream) {
+  if (!q || !k || !workspace || !out) return PDLLM_ERR_NULL;
+  if (prefix_len < 0 || chunk_len <= 0 || query_len <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 ||
+      num_q_heads % num_kv_heads || head_dim <= 0)
+    return PDLLM_ERR_SHAPE;
+  if (head_dim > 256 || query_len > 64) return PDLLM_ERR_UNSUPPORTED;  // limits of the reference scorer
+  float* mx = workspace;
+  float* den = workspace + (int64_t)num_q_heads * query_len;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(evict_maxden_kernel, dim3((unsigned)num_q_heads, (unsigned)query_len), dim3(256), 0, st,
+                     static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), (long)prefix_len,
+                     (long)chunk_len, (long)query_len, num_q_heads, num_kv_heads, head_dim, scale, causal,
+                     mx, den);
+  int rc = launch_status();
+  if (rc != PDLLM_OK) return rc;
+  hipLaunchKernelGGL(evict_chunk_scores_kernel,
+                     dim3((unsigned)num_q_heads, (unsigned)((chunk_len + 63) / 64)), dim3(64),
+                     (size_t)(query_len * head_dim * 4), st, static_cast<const __bf16*>(q),
+                     static_cast<const __bf16*>(k), mx, den, (long)prefix_len, (long)chunk_len,
+                     (long)query_len, num_q_heads, num_kv_heads, head_dim, scale, reduce_mean, out);
+  return launch_status();
+}
+
+extern "C" int pdllm_token_score_pool_group(const float* scores, int64_t n_heads, int64_t n, int32_t pool,
+                                            int32_t kernel, int64_t heads_per_group, float* out,
+                                            pdllm_stream_t stream) {
+  if (!scores || !out) return PDLLM_ERR_NULL;
+  if (n_heads <= 0 || n <= 0 || heads_per_group <= 0 || n_heads % heads_per_group) return PDLLM_ERR_SHAPE;
+  if (pool < 0 || pool > 2) return PDLLM_ERR_DTYPE;
+  if (pool != 0 && kernel < 1) return PDLLM_ERR_SHAPE;
+  const long groups = n_heads / heads_per_group;
+  if (groups > 65535) return PDLLM_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(pool_group_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)groups), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), scores, (long)n_heads, (long)n, pool, kernel,
+                     (long)heads_per_group, out);
+  return launch_status();
+}

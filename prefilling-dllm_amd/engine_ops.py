@@ -1,0 +1,324 @@
+"""Host-side mirror of the tensor-math helpers of the reference engine (fastdllm_engine.py) on top of
+the HIP operators: chunk ranking, token keep-set selection, per-head KV compaction, KV snapshot /
+load, chunk-local KV copy and the confidence-threshold unmask step.  Names, argument meaning and
+error behaviour follow the reference methods (cited per function; ENG = fastdllm_engine.py).
+"""
+from __future__ import annotations
+
+import math
+import threading
+from collections import deque
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from . import ops
+
+PAGE_SIZE = ops.PAGE_SIZE
+
+
+# ------------------------------------------------------------------------------------------
+# PD boundary types (ENG:33-61) -- field for field
+# ------------------------------------------------------------------------------------------
+
+@dataclass
+class FastDLLMEngineOutput:
+    text: str
+    token_ids: List[int]
+    n_diff_steps: int
+
+
+@dataclass
+class DreamPrefillRecord:
+    """Boundary state between prefill and decode (ENG:33-49)."""
+
+    prompt_ids: List[int]
+    prompt_positions: List[int]
+    suffix_positions: List[int]
+    prompt_len: int
+    full_prompt_len: int
+    decode_len: int
+    prompt_page_ids: List[int]
+    block_page_ids: List[int]
+    first_token_id: int
+    last_context_logit: Optional[torch.Tensor]
+    decode_delta_state: Optional[dict]
+    owns_prompt_pages: bool
+    cached_prefix: Optional["_CachedPrefix"] = None
+    kv_mode: str = "full_dense"
+
+
+@dataclass
+class DreamKVSnapshot:
+    """Transferable prompt KV payload (ENG:52-61): per layer [prompt_len, Hkv, d]."""
+
+    prompt_len: int
+    page_size: int
+    kv_mode: str
+    k_by_layer: List[torch.Tensor]
+    v_by_layer: List[torch.Tensor]
+    last_context_logit: Optional[torch.Tensor] = None
+
+
+@dataclass
+class _CachedPrefix:
+    prompt_hash: int
+    page_ids: List[int]
+    prompt_len: int
+    last_context_logit: torch.Tensor
+    ref_count: int = 1
+
+
+class PrefixPageAllocator:
+    """Free-list page allocator with per-page refcounts and hash-keyed prefix sharing (ENG:88-167).
+    Host-side integers only; it stays Python as in the reference."""
+
+    def __init__(self, num_pages: int, page_size: int):
+        self.num_pages = num_pages
+        self.page_size = page_size
+        self.free_pages: deque = deque(range(num_pages))
+        self.page_ref_count: List[int] = [0] * num_pages
+        self.hash_to_prefix: Dict[int, _CachedPrefix] = {}
+        self._lock = threading.RLock()
+
+    @staticmethod
+    def compute_prompt_hash(prompt_ids: List[int]) -> int:
+        import xxhash
+        h = xxhash.xxh64()
+        h.update(np.array(prompt_ids, dtype=np.int64).tobytes())
+        return h.intdigest()
+
+    @property
+    def num_free_pages(self) -> int:
+        with self._lock:
+            return len(self.free_pages)
+
+    def allocate_pages(self, n: int) -> List[int]:
+        with self._lock:
+            if n > len(self.free_pages):
+                raise RuntimeError(f"Cannot allocate {n} pages, only {len(self.free_pages)} free")
+            pages = [self.free_pages.popleft() for _ in range(n)]
+            for p in pages:
+                self.page_ref_count[p] = 1
+            return pages
+
+    def ref_pages(self, pages: List[int]) -> None:
+        with self._lock:
+            for p in pages:
+                self.page_ref_count[p] += 1
+
+    def release_pages(self, pages: List[int]) -> None:
+        with self._lock:
+            for p in pages:
+                self.page_ref_count[p] -= 1
+                if self.page_ref_count[p] == 0:
+                    self.free_pages.append(p)
+
+    def lookup_prefix(self, prompt_ids: List[int]) -> Optional[_CachedPrefix]:
+        with self._lock:
+            return self.hash_to_prefix.get(self.compute_prompt_hash(prompt_ids))
+
+    def register_prefix(self, prompt_ids, page_ids, prompt_len, last_context_logit) -> _CachedPrefix:
+        with self._lock:
+            h = self.compute_prompt_hash(prompt_ids)
+            entry = _CachedPrefix(prompt_hash=h, page_ids=list(page_ids), prompt_len=prompt_len,
+                                  last_context_logit=last_context_logit.detach(), ref_count=0)
+            self.hash_to_prefix[h] = entry
+            return entry
+
+    def release_prefix(self, prompt_ids: List[int]) -> None:
+        with self._lock:
+            entry = self.hash_to_prefix.get(self.compute_prompt_hash(prompt_ids))
+            if entry is not None:
+                entry.ref_count -= 1
+
+    def evict_one(self) -> bool:
+        with self._lock:
+            for h, entry in list(self.hash_to_prefix.items()):
+                if entry.ref_count <= 0:
+                    self.release_pages(entry.page_ids)
+                    del self.hash_to_prefix[h]
+                    return True
+            return False
+
+
+# ------------------------------------------------------------------------------------------
+# chunk ranking (ENG:1199-1204)
+# ------------------------------------------------------------------------------------------
+
+def select_chunks_from_scores(scores: torch.Tensor, topk_chunks: int, keep_first_chunk: bool = False) -> torch.Tensor:
+    """Ranking tail of select_chunks_by_engine: non-finite -> -inf, stable descending order
+    (lowest index first on ties), the top `topk_chunks` of the non-forced chunks plus chunk 0 when
+    keep_first_chunk, returned in ascending chunk order.  scores: device fp32 [n_chunks]."""
+    n = int(scores.numel())
+    if n == 0:
+        return torch.empty(0, dtype=torch.int64, device=scores.device)
+    scores = scores.float().reshape(-1)
+    if keep_first_chunk:
+        rest = scores[1:]
+        k = rest.numel() if int(topk_chunks or 0) <= 0 else min(int(topk_chunks), rest.numel())
+        if k == 0:
+            return torch.zeros(1, dtype=torch.int64, device=scores.device)
+        sel = ops.topk_lowest_index(rest.contiguous(), k, sorted_ascending=True) + 1
+        return torch.cat([torch.zeros(1, dtype=torch.int64, device=scores.device), sel])
+    k = n if int(topk_chunks or 0) <= 0 else min(int(topk_chunks), n)
+    return ops.topk_lowest_index(scores.contiguous(), k, sorted_ascending=True)
+
+
+# ------------------------------------------------------------------------------------------
+# token keep set (ENG:903-927)
+# ------------------------------------------------------------------------------------------
+
+def select_positions_from_token_scores(token_scores: torch.Tensor, *, capacity: int, chunk_len: int,
+                                       keep_high: bool = True, force_keep_first: bool = True) -> torch.Tensor:
+    """_select_positions_from_token_scores with ties broken by lowest index.  token_scores is one
+    row [chunk_len] or a batch [rows, chunk_len] on the device."""
+    keep_count = min(max(1, int(capacity)), int(chunk_len))
+    if token_scores.shape[-1] != chunk_len:
+        head = keep_count // 2
+        tail = keep_count - head
+        keep = sorted(set(list(range(head)) + list(range(chunk_len - tail, chunk_len))))
+        return torch.tensor(keep[:keep_count], device=token_scores.device, dtype=torch.long)
+    return ops.topb_keep_bos(token_scores, capacity, keep_high=keep_high,
+                             force_keep_first=force_keep_first and chunk_len > 0)
+
+
+# ------------------------------------------------------------------------------------------
+# compaction / snapshot / load / chunk-local copy (ENG:525-558, 607-698)
+# ------------------------------------------------------------------------------------------
+
+def compact_prompt_cache_per_head(layer_cache: torch.Tensor, page_ids: torch.Tensor, keep: torch.Tensor) -> int:
+    """One layer, one of K/V: token j of head h <- token keep[h][j]; gather completes before the
+    write (the reference clones), so overlapping source and destination slots are safe."""
+    active_len = int(keep.shape[1])
+    if active_len <= 0:
+        return 0
+    compacted = ops.kv_gather(layer_cache, page_ids, active_len, token_idx=keep)
+    ops.kv_scatter(layer_cache, page_ids, compacted, dst_start=0)
+    return active_len
+
+
+def compact_prompt_cache_per_layer_per_head(kv_cache: torch.Tensor, prompt_page_ids: Sequence[int],
+                                            keep_indices_per_layer_per_head: Sequence[torch.Tensor]) -> int:
+    """_compact_prompt_cache_per_layer_per_head (ENG:607-638) on kv_cache [2, L, pages, P, Hkv, d]."""
+    if not keep_indices_per_layer_per_head:
+        return 0
+    page_ids = torch.as_tensor(list(prompt_page_ids), dtype=torch.int32, device=kv_cache.device)
+    active_len = int(keep_indices_per_layer_per_head[0].shape[1])
+    if active_len <= 0:
+        return 0
+    for layer_idx, keep in enumerate(keep_indices_per_layer_per_head):
+        keep = keep.to(device=kv_cache.device, dtype=torch.long)
+        for kv in range(2):
+            compact_prompt_cache_per_head(kv_cache[kv, layer_idx], page_ids, keep)
+    return active_len
+
+
+def normalize_per_head_keep_indices(keep_indices_per_layer_per_head, *, num_layers: int, num_heads: int,
+                                    full_prompt_len: int, device) -> Tuple[List[torch.Tensor], int]:
+    """Shape / range checks of _normalize_per_head_keep_indices (ENG:560-605)."""
+    if len(keep_indices_per_layer_per_head) != num_layers:
+        raise ValueError("per-head keep index layer count mismatch: "
+                         f"got {len(keep_indices_per_layer_per_head)}, expected {num_layers}")
+    normalized: List[torch.Tensor] = []
+    active_len: Optional[int] = None
+    for layer_idx, layer_keep in enumerate(keep_indices_per_layer_per_head):
+        keep = torch.as_tensor(layer_keep, dtype=torch.long, device=device)
+        if keep.ndim != 2:
+            raise ValueError(f"Layer {layer_idx} keep indices must be [num_heads, active_len], got {tuple(keep.shape)}")
+        if int(keep.shape[0]) != num_heads:
+            raise ValueError(f"Layer {layer_idx} keep head count mismatch: got {keep.shape[0]}, expected {num_heads}")
+        if active_len is None:
+            active_len = int(keep.shape[1])
+        elif int(keep.shape[1]) != active_len:
+            raise ValueError(f"Layer {layer_idx} active length mismatch: got {keep.shape[1]}, expected {active_len}")
+        if keep.numel() > 0:
+            if int(keep.min().item()) < 0 or int(keep.max().item()) >= full_prompt_len:
+                raise ValueError(f"Layer {layer_idx} keep indices are outside full prompt length {full_prompt_len}.")
+        normalized.append(keep.contiguous())
+    return normalized, int(active_len or 0)
+
+
+def snapshot_prompt_cache_per_layer(kv_cache: torch.Tensor, prompt_page_ids: Sequence[int],
+                                    prompt_len: int) -> Tuple[List[torch.Tensor], List[torch.Tensor]]:
+    """_snapshot_prompt_cache_per_layer (ENG:640-662): per layer [prompt_len, Hkv, d] for K and V."""
+    if prompt_len <= 0:
+        return [], []
+    page_ids = torch.as_tensor(list(prompt_page_ids), dtype=torch.int32, device=kv_cache.device)
+    full_k = [ops.kv_gather(kv_cache[0, l], page_ids, int(prompt_len)) for l in range(kv_cache.shape[1])]
+    full_v = [ops.kv_gather(kv_cache[1, l], page_ids, int(prompt_len)) for l in range(kv_cache.shape[1])]
+    return full_k, full_v
+
+
+def load_prompt_cache_per_layer(kv_cache: torch.Tensor, prompt_page_ids: Sequence[int], prompt_len: int,
+                                k_by_layer: Sequence[torch.Tensor], v_by_layer: Sequence[torch.Tensor]) -> None:
+    """_load_prompt_cache_per_layer (ENG:664-698) with its shape checks."""
+    if prompt_len <= 0:
+        return
+    L = int(kv_cache.shape[1])
+    if len(k_by_layer) != L or len(v_by_layer) != L:
+        raise ValueError(f"PD KV snapshot layer count mismatch: k={len(k_by_layer)} v={len(v_by_layer)} expected={L}")
+    page_ids = torch.as_tensor(list(prompt_page_ids), dtype=torch.int32, device=kv_cache.device)
+    expected = (int(prompt_len), int(kv_cache.shape[4]), int(kv_cache.shape[5]))
+    for l, (lk, lv) in enumerate(zip(k_by_layer, v_by_layer)):
+        lk = lk.to(device=kv_cache.device, dtype=kv_cache.dtype)
+        lv = lv.to(device=kv_cache.device, dtype=kv_cache.dtype)
+        if tuple(lk.shape) != expected or tuple(lv.shape) != expected:
+            raise ValueError(f"PD KV snapshot shape mismatch at layer {l}: k={tuple(lk.shape)} "
+                             f"v={tuple(lv.shape)} expected={expected}")
+        ops.kv_scatter(kv_cache[0, l], page_ids, lk)
+        ops.kv_scatter(kv_cache[1, l], page_ids, lv)
+
+
+def snapshot_pd_record_kv(kv_cache: torch.Tensor, record: DreamPrefillRecord, *, page_size: int = PAGE_SIZE,
+                          device="cpu") -> DreamKVSnapshot:
+    """snapshot_pd_record_kv (ENG:700-726): gather the record's prompt KV and move it to `device`."""
+    k, v = snapshot_prompt_cache_per_layer(kv_cache, record.prompt_page_ids, record.prompt_len)
+    ll = record.last_context_logit
+    return DreamKVSnapshot(prompt_len=record.prompt_len, page_size=page_size, kv_mode=record.kv_mode,
+                           k_by_layer=[t.to(device) for t in k], v_by_layer=[t.to(device) for t in v],
+                           last_context_logit=None if ll is None else ll.to(device))
+
+
+def copy_chunk_local_kv_to_prompt_pages(kv_cache: torch.Tensor, *, src_page_ids: Sequence[int],
+                                        dst_page_ids: Sequence[int], src_chunk_start: int, dst_start: int,
+                                        keep_indices_per_layer_per_head: Sequence[torch.Tensor]) -> int:
+    """_copy_chunk_local_kv_to_prompt_pages (ENG:525-558): kept tokens of a chunk prefilled into
+    temporary pages are copied, per layer and KV head, behind dst_start of the request's pages."""
+    if not keep_indices_per_layer_per_head:
+        return 0
+    dev = kv_cache.device
+    src_pages = torch.as_tensor(list(src_page_ids), dtype=torch.int32, device=dev)
+    dst_pages = torch.as_tensor(list(dst_page_ids), dtype=torch.int32, device=dev)
+    keep_count = int(keep_indices_per_layer_per_head[0].shape[1])
+    if keep_count <= 0:
+        return 0
+    for layer_idx, keep in enumerate(keep_indices_per_layer_per_head):
+        keep = keep.to(device=dev, dtype=torch.long)
+        if int(keep.shape[1]) != keep_count:
+            raise ValueError(f"Layer {layer_idx} keep_count mismatch in chunk-local KV copy")
+        for kv in range(2):
+            gathered = ops.kv_gather(kv_cache[kv, layer_idx], src_pages, keep_count, token_idx=keep,
+                                     src_offset=int(src_chunk_start))
+            ops.kv_scatter(kv_cache[kv, layer_idx], dst_pages, gathered, dst_start=int(dst_start))
+    return keep_count
+
+
+# ------------------------------------------------------------------------------------------
+# one denoise step after the model forward (ENG:2143-2157), no host synchronisation
+# ------------------------------------------------------------------------------------------
+
+def denoise_unmask_step(logits: torch.Tensor, block_ids: torch.Tensor, *, mask_token_id: int, threshold: float,
+                        last_context_logit: Optional[torch.Tensor] = None,
+                        shift: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """logits [n_seqs*block_len, vocab] bf16, block_ids [n_seqs, block_len] int64 (updated in place).
+    shift=True applies the Dream logit shift (_shift_logits, ENG:1647-1656) while reading; LLaDA
+    uses shift=False.  Confidence = fp32 max-softmax, token = first argmax (_sample_tokens at
+    temperature 0, ENG:1675-1681); transfer = most confident masked position plus every masked
+    position with confidence >= threshold (ENG:2146-2157).  Returns (transfer mask, masked left)."""
+    n_seqs, block_len = block_ids.shape
+    conf, tok = ops.conf_argmax(logits, block_len, shift=shift, last_logit=last_context_logit)
+    return ops.threshold_unmask(conf.view(n_seqs, block_len), tok.view(n_seqs, block_len), block_ids,
+                                mask_token_id, threshold)

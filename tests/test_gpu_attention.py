@@ -1,0 +1,256 @@
+"""GPU parity of the sparse-prefix attention kernels against the CPU oracle (through the C ABI)."""
+import math
+
+import pytest
+import torch
+
+from oracle import configs, ref_ops
+
+pytestmark = pytest.mark.gpu
+
+TOL_BF16 = 2e-2   # max-abs tolerance of bf16 attention outputs (north star)
+TOL_REL_FP32 = 1e-3
+
+
+def _ops():
+    from prefilling_dllm_amd import ops
+    return ops
+
+
+def run_case(case, dev, *, mask_mode="full", mask=None, rows_per_group=0, num_splits=0, use_ctx_lens=False,
+             sm_scale=None):
+    ops = _ops()
+    d = lambda t: None if t is None else t.to(dev)
+    rp, rs, rl, mr = case.range_tensors()
+    kwargs = dict(max_q_len=case.max_q, max_ctx_len=case.max_ctx, mask_mode=mask_mode, mask=d(mask),
+                  sm_scale=sm_scale, k_scale=d(case.k_scale), v_scale=d(case.v_scale),
+                  rows_per_group=rows_per_group, num_splits=num_splits)
+    if use_ctx_lens:
+        kwargs["context_lens"] = d(torch.tensor([sum(l for _, l in rr) for rr in case.ranges], dtype=torch.int32))
+    else:
+        kwargs["ranges"] = (d(rp), d(rs), d(rl), mr)
+    out = ops.sparse_decode_attention(d(case.q), d(case.k_new), d(case.v_new), d(case.k_cache), d(case.v_cache),
+                                      d(case.block_table), d(case.q_start_loc), **kwargs)
+    torch.cuda.synchronize()
+    return out.float().cpu()
+
+
+def oracle_case(case, *, mask_mode="full", mask=None, sm_scale=None):
+    kc = case.k_cache_ref if case.k_cache_ref is not None else case.k_cache
+    vc = case.v_cache_ref if case.v_cache_ref is not None else case.v_cache
+    return ref_ops.sparse_decode_attention(case.q, case.k_new, case.v_new, kc, vc, case.block_table,
+                                           case.q_start_loc, case.ranges, mask_mode=mask_mode, mask=mask,
+                                           sm_scale=sm_scale)
+
+
+def check(out, ref, tol=TOL_BF16):
+    assert torch.isfinite(out).all()
+    err = (out - ref).abs().max().item()
+    assert err <= tol, f"max abs err {err}"
+    # relative check against the fp32 reference norm (bf16 output rounding dominates)
+    rel = (out - ref).norm() / ref.norm().clamp_min(1e-12)
+    assert rel <= 1e-2, f"relative error {rel}"
+
+
+def test_config1_parity(dev):
+    """BASELINE config 1: 8 x 1025-token chunks in shuffled pages, top-K 4, 96 active rows."""
+    case = configs.config1(seed=1)
+    check(run_case(case, dev), oracle_case(case))
+
+
+@pytest.mark.parametrize("rows", [32, 64, 128, 160, 192, 256])
+@pytest.mark.parametrize("splits", [1, 2, 3])
+def test_row_group_and_split_variants(dev, rows, splits):
+    """Every row-group shape (own / shared row blocks, LDS merge) and the workspace split path on
+    a ragged case: chunks of 300 tokens (not page aligned, partial last tile), 40 active rows."""
+    case = configs.chunked_prefix_case(7, n_req=2, n_chunks=5, chunk_tokens=300, topk=2, q_len=40,
+                                       shared_prefix=False)
+    ref = oracle_case(case)
+    check(run_case(case, dev, rows_per_group=rows, num_splits=splits), ref)
+
+
+@pytest.mark.parametrize("rows", [0, 160, 256])
+def test_config3_shape_small_batch(dev, rows):
+    case = configs.config3_small(seed=3, n_req=2)
+    check(run_case(case, dev, rows_per_group=rows), oracle_case(case))
+
+
+def test_context_lens_path_matches_ranges(dev):
+    """The reference's decode context (first ctx_len tokens of the page table) is the single-range case."""
+    case = configs.chunked_prefix_case(11, n_req=3, n_chunks=1, chunk_tokens=333, topk=1, q_len=32,
+                                       shared_prefix=False)
+    ref = oracle_case(case)
+    check(run_case(case, dev, use_ctx_lens=True), ref)
+    check(run_case(case, dev), ref)
+
+
+def test_mha_group_of_one(dev):
+    case = configs.chunked_prefix_case(5, n_req=2, n_chunks=3, chunk_tokens=257, topk=2, q_len=64, Hq=8, Hkv=8)
+    check(run_case(case, dev), oracle_case(case))
+
+
+def test_causal_and_dense_masks(dev):
+    case = configs.chunked_prefix_case(9, n_req=2, n_chunks=2, chunk_tokens=100, topk=1, q_len=70,
+                                       shared_prefix=False)
+    check(run_case(case, dev, mask_mode="causal"), oracle_case(case, mask_mode="causal"))
+    gen = torch.Generator().manual_seed(0)
+    n = case.q.shape[0]
+    mask = torch.rand(n, n, generator=gen) < 0.5
+    check(run_case(case, dev, mask_mode="dense", mask=mask), oracle_case(case, mask_mode="dense", mask=mask))
+
+
+def test_reference_decoding_test_procedure(dev):
+    """The procedure of the reference's examples/test_dllm_decoding_kernel.py:11-97: 20 sequences of
+    64 active rows over contexts of 81..120 tokens (one page each), block-causal dense mask, checked
+    on every sequence (the reference checks sequence 0 only)."""
+    torch.manual_seed(114514)
+    seq = torch.tensor([64] * 20, dtype=torch.int32)
+    ctx = torch.tensor([119, 110, 81, 114, 112, 119, 110, 81, 114, 112, 119, 110, 81, 114, 112, 120, 111, 82, 115,
+                        113], dtype=torch.int32)
+    n = int(seq.sum())
+    q = torch.randn(n, 28, 128).to(torch.bfloat16)
+    k = torch.randn(n, 4, 128).to(torch.bfloat16)
+    v = torch.randn(n, 4, 128).to(torch.bfloat16)
+    k_cache = torch.randn(20, 256, 4, 128).to(torch.bfloat16)
+    v_cache = torch.randn(20, 256, 4, 128).to(torch.bfloat16)
+    bt = torch.arange(20, dtype=torch.int32).view(20, 1)
+    cu = torch.cat([torch.zeros(1, dtype=torch.int32), torch.cumsum(seq, 0).to(torch.int32)])
+    mask = torch.zeros(n, n, dtype=torch.bool)
+    for i in range(20):
+        s = int(cu[i])
+        for b in range(2):
+            mask[s + 32 * b:s + 32 * b + 32, s:s + 32 * b + 32] = True
+    ops = _ops()
+    out = torch.empty(n, 28, 128, dtype=torch.bfloat16, device=dev)
+    scale = 1.0 / math.sqrt(128)
+    ops.diffusion_lm_parallel_flash_decoding(q.to(dev), k.to(dev), v.to(dev), out, "torch.bfloat16",
+                                             k_cache.to(dev), v_cache.to(dev), bt.to(dev), cu.to(dev),
+                                             (seq + ctx).to(dev), int((seq + ctx).max()), 64, 1.0, 1.0,
+                                             diffusion_blk_sz=32, sm_scale=scale, mask=mask.to(dev))
+    torch.cuda.synchronize()
+    ranges = [[(0, int(c))] for c in ctx]
+    ref = ref_ops.sparse_decode_attention(q, k, v, k_cache, v_cache, bt, cu, ranges, mask_mode="dense", mask=mask,
+                                          sm_scale=scale)
+    # N(0,1) inputs give outputs of magnitude ~1; bf16 rounding of O dominates
+    check(out.float().cpu(), ref, tol=3e-2)
+
+
+def test_fully_masked_rows_give_zeros(dev):
+    case = configs.chunked_prefix_case(2, n_req=1, n_chunks=1, chunk_tokens=64, topk=1, q_len=32)
+    case.ranges = [[]]  # no visible prefix
+    n = case.q.shape[0]
+    mask = torch.ones(n, n, dtype=torch.bool)
+    mask[5, :] = False
+    ops = _ops()
+    d = lambda t: t.to(dev)
+    out = ops.sparse_decode_attention(d(case.q), d(case.k_new), d(case.v_new), None, None, None,
+                                      d(case.q_start_loc), max_q_len=32, max_ctx_len=0, mask_mode="dense",
+                                      mask=d(mask)).float().cpu()
+    ref = oracle_case(case, mask_mode="dense", mask=mask)
+    assert out[5].abs().max() == 0
+    check(out, ref)
+
+
+def test_fp8_pages_with_per_page_scale(dev):
+    """BASELINE config 5 shape (MHA, fp8 e4m3 pages, fp32 scale per page) at reduced size; the
+    oracle sees float(e4m3) * scale rounded to bf16, i.e. exactly what the kernel dequantises."""
+    case = configs.config5_small(seed=4, n_req=2, n_chunks=6, topk=3)
+    check(run_case(case, dev), oracle_case(case))
+
+
+def test_fp8_codes_decode_like_torch(dev):
+    """All 256 e4m3 codes through the kernel's dequantisation == torch.float8_e4m3fn -> float."""
+    ops = _ops()
+    codes = torch.arange(0x7f, dtype=torch.uint8)  # every positive code (0x7f is NaN); mean is far from 0
+    n = codes.numel()
+    # one key per code: V row = the code in every element, K = 0 so softmax is uniform over n keys
+    Hkv, dd = 1, 128
+    pages = (n + 255) // 256
+    v8 = torch.zeros(pages * 256, Hkv, dd, dtype=torch.uint8)
+    v8[:n] = codes.view(n, 1, 1)
+    k8 = torch.zeros_like(v8)
+    scale = torch.tensor([0.5] * pages, dtype=torch.float32)
+    q = torch.zeros(32, 1, dd, dtype=torch.bfloat16)
+    knew = torch.zeros(32, 1, dd, dtype=torch.bfloat16)
+    # active block fully masked out so only the cache is averaged
+    mask = torch.zeros(32, 32, dtype=torch.bool)
+    bt = torch.arange(pages, dtype=torch.int32).view(1, pages)
+    out = ops.sparse_decode_attention(q.to(dev), knew.to(dev), knew.to(dev),
+                                      k8.view(pages, 256, Hkv, dd).view(torch.float8_e4m3fn).to(dev),
+                                      v8.view(pages, 256, Hkv, dd).view(torch.float8_e4m3fn).to(dev), bt.to(dev),
+                                      torch.tensor([0, 32], dtype=torch.int32, device=dev), max_q_len=32,
+                                      max_ctx_len=n, context_lens=torch.tensor([n], dtype=torch.int32, device=dev),
+                                      mask_mode="dense", mask=mask.to(dev), k_scale=scale.to(dev),
+                                      v_scale=scale.to(dev)).float().cpu()
+    vals = (codes.view(torch.float8_e4m3fn).float() * 0.5).to(torch.bfloat16).float()
+    expect = vals.mean().item()
+    assert abs(out[0, 0, 0].item() - expect) <= 2e-2 * max(1.0, abs(expect))
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_chunk_prefill_block_diagonal(dev, causal):
+    """BASELINE config 4 shape at reduced size: independent chunks of ragged length, causal inside a
+    chunk, K/V written to shuffled pages through a slot mapping."""
+    gen = torch.Generator().manual_seed(21)
+    lens = [257, 64, 1, 130, 300]
+    n = sum(lens)
+    Hq, Hkv, dd = 28, 4, 128
+    q = (torch.randn(n, Hq, dd, generator=gen)).to(torch.bfloat16)
+    k = (torch.randn(n, Hkv, dd, generator=gen)).to(torch.bfloat16)
+    v = (torch.randn(n, Hkv, dd, generator=gen)).to(torch.bfloat16)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    n_pages = (n + 255) // 256 + 2
+    page_ids = torch.randperm(n_pages, generator=gen)[:(n + 255) // 256].tolist()
+    slots = ref_ops.slot_mapping(page_ids, n)
+    slots[10] = -1  # a skipped token
+    ops = _ops()
+    kc = torch.zeros(n_pages, 256, Hkv, dd, dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    out = ops.chunk_prefill_attention(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), max_seqlen=max(lens),
+                                      causal=causal, k_cache=kc, v_cache=vc, slot_mapping=slots.to(dev))
+    torch.cuda.synchronize()
+    ref = ref_ops.chunk_prefill_attention(q, k, v, cu, causal=causal)
+    check(out.float().cpu(), ref, tol=3e-2)
+    kc_ref = torch.zeros(n_pages, 256, Hkv, dd, dtype=torch.bfloat16)
+    vc_ref = torch.zeros_like(kc_ref)
+    ref_ops.store_kvcache(k, v, kc_ref, vc_ref, slots)
+    assert torch.equal(kc.cpu(), kc_ref) and torch.equal(vc.cpu(), vc_ref)
+
+
+def test_permuting_pages_leaves_output_unchanged(dev):
+    """Size-independent property: the physical page order is irrelevant (same logical tokens)."""
+    case = configs.chunked_prefix_case(13, n_req=1, n_chunks=4, chunk_tokens=512, topk=4, q_len=32)
+    out1 = run_case(case, dev)
+    perm = torch.randperm(case.k_cache.shape[0], generator=torch.Generator().manual_seed(1))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(perm.numel())
+    case.k_cache = case.k_cache[perm]
+    case.v_cache = case.v_cache[perm]
+    case.block_table = inv[case.block_table.long()].to(torch.int32)
+    out2 = run_case(case, dev)
+    assert torch.equal(out1, out2)
+
+
+def test_value_of_ones_gives_ones(dev):
+    """Rows of the softmax sum to one: V == 1 everywhere => O == 1 (up to bf16 rounding of P)."""
+    case = configs.config3_small(seed=5, n_req=1)
+    case.v_cache = torch.ones_like(case.v_cache)
+    case.v_new = torch.ones_like(case.v_new)
+    out = run_case(case, dev)
+    assert (out - 1.0).abs().max() <= 1e-2
+
+
+def test_error_codes(dev):
+    ops = _ops()
+    q = torch.zeros(32, 4, 64, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(NotImplementedError):
+        ops.sparse_decode_attention(q, q, q, None, None, None, torch.tensor([0, 32], dtype=torch.int32, device=dev),
+                                    max_q_len=32, max_ctx_len=0)
+    q = torch.zeros(32, 6, 128, dtype=torch.bfloat16, device=dev)
+    k = torch.zeros(32, 4, 128, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(ValueError):
+        ops.sparse_decode_attention(q, k, k, None, None, None, torch.tensor([0, 32], dtype=torch.int32, device=dev),
+                                    max_q_len=32, max_ctx_len=0)
+    with pytest.raises(ValueError):
+        ops.sparse_decode_attention(q.cpu(), k.cpu(), k.cpu(), None, None, None,
+                                    torch.tensor([0, 32], dtype=torch.int32), max_q_len=32, max_ctx_len=0)

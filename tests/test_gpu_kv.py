@@ -1,0 +1,162 @@
+"""GPU parity of the paged KV data movement (store / load / gather / scatter / compaction)."""
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import ref_ops
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _ops():
+    from prefilling_dllm_amd import ops
+    return ops
+
+
+def test_store_reference_procedure(dev):
+    """examples/test_dllm_kv_cache_store.py:8-43 of the reference: 20 sequences, contexts 81..120,
+    32 active rows each mapped to -1, cache (307, 256, 4, 128) bf16, seed 114514."""
+    torch.manual_seed(114514)
+    ctx = [119, 110, 81, 114, 112, 119, 110, 81, 114, 112, 119, 110, 81, 114, 112, 120, 111, 82, 115, 113]
+    total = [c + 32 for c in ctx]
+    k = torch.randn(sum(total), 4, 128).to(torch.bfloat16)
+    v = torch.randn(sum(total), 4, 128).to(torch.bfloat16)
+    slots = []
+    for i, c in enumerate(ctx):
+        slots.extend(range(i * 256, i * 256 + c))
+        slots.extend([-1] * 32)
+    slots = torch.tensor(slots, dtype=torch.int64)
+    kc = torch.zeros(307, 256, 4, 128, dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    _ops().store_kvcache_unified_layout(k.to(dev), v.to(dev), kc, vc, slots.to(dev), model_type="diffusion_lm")
+    torch.cuda.synchronize()
+    start = 0
+    for i, (l, c) in enumerate(zip(total, ctx)):
+        assert torch.equal(kc[i, :c].cpu(), k[start:start + c])
+        assert torch.equal(vc[i, :c].cpu(), v[start:start + c])
+        assert kc[i, c:].abs().max() == 0  # masked (-1) rows were not written
+        start += l
+    kc_ref = torch.zeros(307, 256, 4, 128, dtype=torch.bfloat16)
+    vc_ref = torch.zeros_like(kc_ref)
+    ref_ops.store_kvcache(k, v, kc_ref, vc_ref, slots)
+    assert torch.equal(kc.cpu(), kc_ref) and torch.equal(vc.cpu(), vc_ref)
+
+
+def test_store_then_load_reference_fixture(dev):
+    """examples/test_dllm_kv_cache_load.py:28-65 with the reference's slot-mapping fixture
+    (examples/mimic_data/mimic_slot_mapping.py, committed as run-length JSON)."""
+    with open(os.path.join(GOLDEN, "mimic_slot_mapping.json")) as f:
+        fx = json.load(f)
+    slots = []
+    for value, start, count in fx["runs"]:
+        slots.extend([-1] * count if value == "skip" else range(start, start + count))
+    assert len(slots) == fx["length"]
+    torch.manual_seed(114514)
+    seq = [64, 64, 32, 64, 64, 32, 64, 32, 64, 64, 32, 64, 64, 64, 64, 64, 32, 32, 64, 64]
+    ctx = [119, 110, 81, 114, 112, 119, 110, 81, 114, 112, 119, 110, 81, 114, 112, 120, 111, 82, 115, 113]
+    assert sum(seq) == len(slots)
+    n_pages = 1342
+    k_cache = torch.randn(n_pages, 256, 4, 128).to(torch.bfloat16)
+    v_cache = torch.randn(n_pages, 256, 4, 128).to(torch.bfloat16)
+    k_new = torch.randn(sum(seq), 4, 128).to(torch.bfloat16)
+    v_new = torch.randn(sum(seq), 4, 128).to(torch.bfloat16)
+    bt = torch.arange(20, dtype=torch.int32).view(20, 1)
+    ops = _ops()
+    kc, vc = k_cache.to(dev), v_cache.to(dev)
+    slots_t = torch.tensor(slots, dtype=torch.int64)
+    ops.store_kvcache_unified_layout(k_new.to(dev), v_new.to(dev), kc, vc, slots_t.to(dev), model_type="diffusion_lm")
+    ref_ops.store_kvcache(k_new, v_new, k_cache, v_cache, slots_t)
+    torch.cuda.synchronize()
+    assert torch.equal(kc.cpu(), k_cache) and torch.equal(vc.cpu(), v_cache)
+
+    class Seq:
+        diffusion_block_size = 32
+
+    class Ctx:
+        pass
+
+    c = Ctx()
+    c.block_tables = bt.to(dev)
+    c.context_lens = torch.tensor(ctx, dtype=torch.int32, device=dev)
+    c.seq_lens_ts = torch.tensor(seq, dtype=torch.int32, device=dev)
+    c.seq_lens = seq
+    c.seqs = [Seq()]
+    cu = lambda x: torch.tensor([0] + list(torch.tensor(x).cumsum(0)), dtype=torch.int32, device=dev)
+    c.cu_seqlens_q = cu(seq)
+    c.cu_seqlens_k = cu([a + b for a, b in zip(seq, ctx)])
+    k_comb, v_comb = ops.load_kvcache(kc, vc, c, k_new.to(dev), v_new.to(dev))
+    torch.cuda.synchronize()
+    k_ref, v_ref = ref_ops.load_kvcache(k_cache, v_cache, bt, ctx, seq, k_new, v_new)
+    assert torch.equal(k_comb.cpu(), k_ref) and torch.equal(v_comb.cpu(), v_ref)
+
+
+def test_slot_mapping_matches_closed_form(dev):
+    pages = [7, 3, 11, 0, 5]
+    got = _ops().slot_mapping_from_pages(torch.tensor(pages, device=dev), 700, start_token=300).cpu()
+    assert torch.equal(got, ref_ops.slot_mapping(pages, 700, 300))
+    # tokens beyond the page list are not mapped
+    got = _ops().slot_mapping_from_pages(torch.tensor(pages[:2], device=dev), 600).cpu()
+    assert (got[512:] == -1).all() and torch.equal(got[:512], ref_ops.slot_mapping(pages, 512))
+
+
+def test_gather_scatter_roundtrip_and_snapshot(dev):
+    gen = torch.Generator().manual_seed(3)
+    n_pages, Hkv, d = 12, 4, 128
+    cache = torch.randn(n_pages, 256, Hkv, d, generator=gen).to(torch.bfloat16)
+    page_ids = torch.randperm(n_pages, generator=gen)[:5]
+    prompt_len = 1100
+    ops = _ops()
+    snap = ops.kv_gather(cache.to(dev), page_ids.to(dev), prompt_len).cpu()
+    assert torch.equal(snap, ref_ops.gather_tokens(cache, page_ids, torch.arange(prompt_len)))
+    # load into fresh pages of another cache and read back
+    cache2 = torch.zeros_like(cache).to(dev)
+    page_ids2 = torch.randperm(n_pages, generator=gen)[:5]
+    ops.kv_scatter(cache2, page_ids2.to(dev), snap.to(dev))
+    back = ops.kv_gather(cache2, page_ids2.to(dev), prompt_len).cpu()
+    assert torch.equal(back, snap)
+    ref2 = torch.zeros_like(cache)
+    ref_ops.scatter_tokens(ref2, page_ids2, snap)
+    assert torch.equal(cache2.cpu(), ref2)
+
+
+def test_per_head_compaction_matches_reference_order(dev):
+    """fastdllm_engine.py:607-638: gather with per-head keep lists, rewrite into the first slots."""
+    gen = torch.Generator().manual_seed(5)
+    n_pages, Hkv, d = 10, 4, 128
+    cache = torch.randn(n_pages, 256, Hkv, d, generator=gen).to(torch.bfloat16)
+    page_ids = torch.randperm(n_pages, generator=gen)[:6]
+    full_len, keep_n = 1400, 520
+    keep = torch.stack([torch.sort(torch.randperm(full_len, generator=gen)[:keep_n]).values for _ in range(Hkv)])
+    ops = _ops()
+    dc = cache.to(dev)
+    from prefilling_dllm_amd import engine_ops
+    engine_ops.compact_prompt_cache_per_head(dc, page_ids.to(dev), keep.to(dev))
+    torch.cuda.synchronize()
+    ref = cache.clone()
+    ref_ops.compact_per_head(ref, page_ids, keep)
+    assert torch.equal(dc.cpu(), ref)
+
+
+def test_fp8_store_matches_torch_cast(dev):
+    gen = torch.Generator().manual_seed(8)
+    n, Hkv, d, n_pages = 600, 4, 128, 4
+    k = torch.randn(n, Hkv, d, generator=gen).to(torch.bfloat16)
+    v = torch.randn(n, Hkv, d, generator=gen).to(torch.bfloat16)
+    page_ids = [2, 0, 3]
+    slots = ref_ops.slot_mapping(page_ids, n)
+    ks = torch.tensor([0.01, 0.02, 0.013, 0.017])
+    vs = torch.tensor([0.011, 0.009, 0.02, 0.015])
+    kc = torch.zeros(n_pages, 256, Hkv, d, dtype=torch.float8_e4m3fn, device=dev)
+    vc = torch.zeros_like(kc)
+    _ops().store_kvcache_unified_layout(k.to(dev), v.to(dev), kc, vc, slots.to(dev), k_scale=ks.to(dev),
+                                        v_scale=vs.to(dev))
+    torch.cuda.synchronize()
+    page_of = (slots // 256).long()
+    kq = (k.float() / ks[page_of].view(-1, 1, 1)).clamp(-448, 448).to(torch.float8_e4m3fn)
+    vq = (v.float() / vs[page_of].view(-1, 1, 1)).clamp(-448, 448).to(torch.float8_e4m3fn)
+    got_k = kc.view(-1, Hkv, d)[slots.long().to(dev)].cpu().view(torch.uint8)
+    got_v = vc.view(-1, Hkv, d)[slots.long().to(dev)].cpu().view(torch.uint8)
+    assert torch.equal(got_k, kq.view(torch.uint8)) and torch.equal(got_v, vq.view(torch.uint8))

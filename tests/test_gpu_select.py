@@ -1,0 +1,210 @@
+"""GPU parity of scoring / top-K / eviction / unmask / rope kernels against the CPU oracle."""
+import pytest
+import torch
+
+from oracle import configs, ref_ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from prefilling_dllm_amd import ops
+    return ops
+
+
+def test_selfinfo_and_chunk_topk_config2(dev):
+    """BASELINE config 2 scoring: [32 chunks, 4 draft tokens, vocab 152064] bf16 logits -> per chunk
+    summed log-probability of the labels -> top-4 chunk indices, bit exact."""
+    logits, labels = configs.draft_logits(seed=0)
+    ops = _ops()
+    lp = ops.selfinfo_logprob(logits.reshape(-1, logits.shape[-1]).to(dev), labels.reshape(-1).to(dev)).cpu()
+    lp_ref = ref_ops.selfinfo_logprob(logits.reshape(-1, logits.shape[-1]), labels.reshape(-1))
+    assert (lp - lp_ref).abs().max() <= 2e-5 * lp_ref.abs().max()
+    for mean in (False, True):
+        sc = ops.chunk_scores_from_logits(logits.to(dev), labels.to(dev), mean=mean)
+        sc_ref = ref_ops.chunk_scores(logits, labels, mean=mean)
+        assert (sc.cpu() - sc_ref).abs().max() <= 1e-4
+        idx = ops.topk_lowest_index(sc, 4).cpu().tolist()
+        assert idx == ref_ops.topk_lowest_index(sc_ref.tolist(), 4)
+        # the separation of the scores around the cut must exceed the reduction error
+        srt = sorted(sc_ref.tolist(), reverse=True)
+        assert srt[3] - srt[4] > 1e-3
+
+
+def test_selfinfo_ragged_vocab_and_bad_label(dev):
+    gen = torch.Generator().manual_seed(2)
+    logits = (torch.randn(5, 1003, generator=gen) * 3).to(torch.bfloat16)  # rows not 16-byte aligned
+    labels = torch.tensor([0, 1002, 17, -1, 5000])
+    got = _ops().selfinfo_logprob(logits.to(dev), labels.to(dev)).cpu()
+    ref = ref_ops.selfinfo_logprob(logits[:3], labels[:3])
+    assert (got[:3] - ref).abs().max() <= 1e-5 * ref.abs().max() + 1e-6
+    assert torch.isinf(got[3]) and got[3] < 0 and torch.isinf(got[4]) and got[4] < 0
+
+
+def test_topk_ties_and_nonfinite(dev):
+    ops = _ops()
+    s = torch.tensor([1.0, 3.0, 3.0, float("nan"), 2.0, 3.0, float("inf"), -float("inf"), 2.0])
+    for k in range(0, 10):
+        if k == 0:
+            continue
+        got = ops.topk_lowest_index(s.to(dev), k).cpu().tolist()
+        assert got == ref_ops.topk_lowest_index(s.tolist(), k), k
+        got_r = ops.topk_lowest_index(s.to(dev), k, sorted_ascending=False).cpu().tolist()
+        assert got_r == ref_ops.topk_lowest_index(s.tolist(), k, sorted_ascending=False), k
+    # many equal scores: the selection is the k lowest indices
+    z = torch.zeros(64)
+    assert ops.topk_lowest_index(z.to(dev), 16).cpu().tolist() == list(range(16))
+    # batched rows
+    gen = torch.Generator().manual_seed(1)
+    b = torch.randint(0, 5, (7, 33), generator=gen).float()
+    got = ops.topk_lowest_index(b.to(dev), 8).cpu()
+    for r in range(7):
+        assert got[r].tolist() == ref_ops.topk_lowest_index(b[r].tolist(), 8)
+
+
+def test_topk_long_rows_radix(dev):
+    gen = torch.Generator().manual_seed(4)
+    s = torch.randint(0, 50, (3, 5000), generator=gen).float()  # heavy ties
+    got = _ops().topk_lowest_index(s.to(dev), 700).cpu()
+    for r in range(3):
+        assert got[r].tolist() == ref_ops.topk_lowest_index(s[r].tolist(), 700)
+
+
+def test_eviction_config2_bit_exact(dev):
+    """BASELINE config 2 eviction: probabilities [28, 64, 1025] per chunk, column sums over heads
+    and queries, BOS + top-255 kept, indices bit exact."""
+    probs = configs.eviction_probs(seed=0, n_chunks=3)
+    ops = _ops()
+    sc = ops.evict_colsum(probs.to(dev))
+    sc_ref = ref_ops.evict_colsum(probs)
+    assert torch.equal(sc.cpu(), sc_ref)                    # same summation order => same bits
+    assert (sc_ref[:, 0].sum(-1) - 28 * 64).abs().max() < 1e-1  # rows of a softmax sum to one
+    keep = ops.topb_keep_bos(sc[:, 0], 256).cpu()
+    for c in range(3):
+        ref = ref_ops.select_positions_from_token_scores(sc_ref[c, 0], capacity=256, chunk_len=1025)
+        assert keep[c].tolist() == ref.tolist()
+        assert keep[c, 0] == 0
+    # per-KV-head grouping (7 q-heads per group)
+    g = ops.evict_colsum(probs.to(dev), heads_per_group=7).cpu()
+    assert torch.equal(g, ref_ops.evict_colsum(probs, heads_per_group=7))
+
+
+def test_topb_degenerate_branches(dev):
+    from prefilling_dllm_amd import engine_ops
+    gen = torch.Generator().manual_seed(6)
+    s = torch.rand(40, generator=gen)
+    s[7] = s[9] = s[3]  # ties
+    cases = [dict(capacity=1), dict(capacity=0), dict(capacity=39), dict(capacity=40), dict(capacity=100),
+             dict(capacity=10), dict(capacity=10, keep_high=False), dict(capacity=10, force_keep_first=False),
+             dict(capacity=10, keep_high=False, force_keep_first=False)]
+    for kw in cases:
+        got = engine_ops.select_positions_from_token_scores(s.to(dev), chunk_len=40, **kw).cpu().tolist()
+        ref = ref_ops.select_positions_from_token_scores(s, chunk_len=40, **kw).tolist()
+        assert got == ref, kw
+    # wrong-length scores -> head/tail fallback
+    got = engine_ops.select_positions_from_token_scores(s[:5].to(dev), capacity=6, chunk_len=40).cpu().tolist()
+    assert got == ref_ops.select_positions_from_token_scores(s[:5], capacity=6, chunk_len=40).tolist()
+
+
+def test_query_to_chunk_scores(dev):
+    gen = torch.Generator().manual_seed(9)
+    prefix, chunk, ql = 3, 300, 8
+    S = prefix + chunk + ql
+    q = torch.randn(S, 28, 128, generator=gen).to(torch.bfloat16)
+    k = torch.randn(S, 4, 128, generator=gen).to(torch.bfloat16)
+    scale = 128 ** -0.5
+    ops = _ops()
+    for mask in ("causal", "full"):
+        for red in ("sum", "mean"):
+            got = ops.query_to_chunk_attention_scores(q.to(dev), k.to(dev), prefix_len=prefix, chunk_len=chunk,
+                                                      query_len=ql, scale=scale, reduce_mode=red,
+                                                      attention_mask=mask).cpu()
+            ref = ref_ops.chunk_attention_head_scores(q, k, prefix_len=prefix, chunk_len=chunk, query_len=ql,
+                                                      scale=scale, reduce_mode=red, attention_mask=mask)
+            assert (got - ref).abs().max() <= 1e-4 * ref.abs().max() + 1e-7
+    with pytest.raises(ValueError):
+        ops.query_to_chunk_attention_scores(q.to(dev), k.to(dev), prefix_len=prefix, chunk_len=chunk - 1,
+                                            query_len=65, scale=scale)
+
+
+def test_pool_and_group(dev):
+    gen = torch.Generator().manual_seed(10)
+    s = torch.rand(28, 1025, generator=gen)
+    ops = _ops()
+    for pooling in ("none", "maxpool", "avgpool"):
+        got = ops.token_score_pool_group(s.to(dev), pooling, 7, num_kv_heads=4).cpu()
+        ref = ref_ops.token_score_pool_group(s, pooling, 7, num_kv_heads=4)
+        assert (got - ref).abs().max() <= 1e-6, pooling
+    got = ops.token_score_pool_group(s.to(dev), "maxpool", 7).cpu()
+    assert torch.equal(got, ref_ops.token_score_pool_group(s, "maxpool", 7))
+
+
+def test_unmask_config5_bit_exact(dev):
+    """BASELINE config 5 unmask: bf16 logits [4*32, 126464], fp32 max-softmax >= 0.9 unmasks with the
+    argmax token (LLaDA: no logit shift); decisions and tokens bit exact."""
+    logits = configs.unmask_logits(seed=0)
+    ops = _ops()
+    conf, tok = ops.conf_argmax(logits.to(dev), 32)
+    conf_ref, tok_ref = ref_ops.sample_tokens(logits)
+    assert torch.equal(tok.cpu(), tok_ref)
+    # fp32 sums in a different order and the hardware exp2: confidences agree to ~1e-5 relative
+    assert (conf.cpu() - conf_ref).abs().max() <= 5e-5
+    assert ((conf_ref - 0.9).abs() > 1e-3).all()  # no row sits on the threshold
+    mask_id = 126336
+    block = torch.full((4, 32), mask_id, dtype=torch.int64)
+    block[:, 0] = 11  # already decoded positions stay
+    block[2, 5] = 12
+    dblock = block.to(dev)
+    from prefilling_dllm_amd import engine_ops
+    transfer, left = engine_ops.denoise_unmask_step(logits.to(dev), dblock, mask_token_id=mask_id, threshold=0.9,
+                                                    shift=False)
+    for b in range(4):
+        nb, tr = ref_ops.threshold_unmask(block[b], conf_ref.view(4, 32)[b], tok_ref.view(4, 32)[b], mask_id, 0.9)
+        assert torch.equal(dblock[b].cpu(), nb)
+        assert torch.equal(transfer[b].cpu(), tr)
+        assert int(left[b]) == int((nb == mask_id).sum())
+        assert tr.sum() >= 1
+
+
+def test_unmask_with_dream_shift(dev):
+    gen = torch.Generator().manual_seed(12)
+    vocab, L = 4096, 32
+    logits = (torch.randn(2 * L, vocab, generator=gen) * 4).to(torch.bfloat16)
+    last = (torch.randn(2, vocab, generator=gen) * 4).to(torch.bfloat16)
+    conf, tok = _ops().conf_argmax(logits.to(dev), L, shift=True, last_logit=last.to(dev))
+    for b in range(2):
+        sh = ref_ops.shift_logits(logits[b * L:(b + 1) * L], last[b])
+        c_ref, t_ref = ref_ops.sample_tokens(sh)
+        assert torch.equal(tok[b * L:(b + 1) * L].cpu(), t_ref)
+        assert (conf[b * L:(b + 1) * L].cpu() - c_ref).abs().max() <= 5e-5
+    conf2, tok2 = _ops().conf_argmax(logits.to(dev), L, shift=True)
+    sh = ref_ops.shift_logits(logits[:L], None)
+    assert torch.equal(tok2[:L].cpu(), ref_ops.sample_tokens(sh)[1])
+
+
+def test_argmax_first_index_on_ties(dev):
+    logits = torch.zeros(3, 70000, dtype=torch.bfloat16)
+    logits[0, 69999] = 5; logits[0, 123] = 5
+    logits[1, 40000] = 2; logits[1, 40001] = 2
+    conf, tok = _ops().conf_argmax(logits.to(dev), 1)
+    assert tok.cpu().tolist() == [123, 40000, 0]
+    assert torch.equal(tok.cpu(), ref_ops.sample_tokens(logits)[1])
+
+
+def test_unmask_all_below_threshold_moves_exactly_one(dev):
+    conf = torch.tensor([[0.2, 0.5, 0.5, 0.1]])
+    tok = torch.tensor([[7, 8, 9, 10]])
+    block = torch.full((1, 4), 99, dtype=torch.int64, device=dev)
+    tr, left = _ops().threshold_unmask(conf.to(dev), tok.to(dev), block, 99, 0.9)
+    assert block.cpu().tolist() == [[99, 8, 99, 99]] and int(left[0]) == 3
+    nb, _ = ref_ops.threshold_unmask(torch.full((4,), 99), conf[0], tok[0], 99, 0.9)
+    assert nb.tolist() == [99, 8, 99, 99]
+
+
+def test_rope_matches_reference_formula(dev):
+    gen = torch.Generator().manual_seed(14)
+    cs = ref_ops.rope_cos_sin_cache(128, 40000, base=1000000.0)
+    x = torch.randn(100, 4, 128, generator=gen).to(torch.bfloat16)
+    pos = torch.randint(0, 40000, (100,), generator=gen)
+    got = _ops().rope_inplace(x.clone().to(dev), pos.to(dev), cs.to(dev)).cpu()
+    assert torch.equal(got, ref_ops.apply_rope(x, pos, cs))
