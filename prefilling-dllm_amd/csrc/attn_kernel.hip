@@ -586,13 +586,16 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
     using N2 = std::integral_constant<int, 2>;
     using Dual = std::integral_constant<bool, NB == 4>;
     using Single = std::integral_constant<bool, false>;
-    dma_begin(t + 1, sb_next, buf ^ 1, has_next);
-    if (HAS_A) {
-      pass(gen_tag, N2{}, Dual{}, I0{}, true, 0, bufoff, nvalid, active, a0, buf);
-      pass(gen_tag, N2{}, Dual{}, I8{}, true, 2, bufoff, nvalid, active, a0, buf);
-    } else {
+    if (has_next) {
+      // the whole copy of the next tile is issued up front (the copy instructions are scheduling
+      // boundaries; spreading them through the MFMA loops measured slower)
+      dma_begin(t + 1, sb_next, buf ^ 1, true);
       dma_offsets(I0{}, I8{});
       dma_all();
+    }
+    if (HAS_A) {
+      pass(gen_tag, N2{}, Dual{}, I16{}, true, 0, bufoff, nvalid, active, a0, buf);
+      pass(gen_tag, N2{}, Dual{}, I16{}, true, 2, bufoff, nvalid, active, a0, buf);
     }
     if (NB == 1) pass(gen_tag, N1{}, Single{}, I16{}, false, kb0, bufoff, nvalid, active, a0, buf);
     if (NB == 2) pass(gen_tag, N2{}, Single{}, I16{}, false, kb0, bufoff, nvalid, active, a0, buf);
@@ -829,6 +832,7 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   for (int ji = 0; ji < 6; ++ji) {
     const int J = js[ji];
     if (d->rows_per_group && d->rows_per_group != 32 * J) continue;
+    if (!d->rows_per_group && J == 8) continue;  // two full row blocks per wave spill registers: only on request
     const long row_tiles = (nblk + J - 1) / J;
     const int max_splits = prefill ? 1 : 16;
     for (int S = 1; S <= max_splits; ++S) {
