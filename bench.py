@@ -23,6 +23,9 @@ if ROOT not in sys.path:
 
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
 PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
+# HBM bytes of one attn_fwd_kernel launch of this workload, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.0,
+# WRITE_SIZE x 1.0 after calibration on a 1 GiB copy): profiles/attn_fwd_kernel_c3_decode_hbm_traffic.txt
+MEASURED_TRAFFIC_BYTES = {(Q_LEN_DEFAULT := 160): 90.00e6}
 
 HQ, HKV, D, PAGE = 28, 4, 128, 256
 LAYERS, N_REQ, N_CHUNKS, TOPK, CHUNK_TOKENS = 28, 8, 32, 8, 512
@@ -126,6 +129,9 @@ def main():
     ap.add_argument("--num-splits", type=int, default=0, help="override the KV split count (tuning)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary shapes")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="also run a plain device copy of this many MiB (a kernel of known traffic, used to "
+                         "scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is single-GPU (one MI355X); --gpus must be 1", file=sys.stderr)
@@ -139,6 +145,15 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.copy_calibration > 0:
+        n = args.copy_calibration << 20
+        src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     w = build_workload(torch, dev)
     preps = prepare(ops, w, args.rows_per_group, args.num_splits)
@@ -186,7 +201,8 @@ def main():
                                "response rows) over 8x512 non-contiguous KV tokens in 256-token pages, GQA 28/4 d128",
                    "rows_per_workgroup": rows, "kv_splits": splits},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                     "frac": tflops / PEAK_BF16_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(w["q_len"]) if not (args.rows_per_group or args.num_splits) else None,
                      "kernel": "attn_fwd_kernel", "avg_launch_us": launch_s * 1e6,
                      "algorithmic_flops_per_launch": fl, "algorithmic_bytes_per_launch": by},
         "hbm": {"achieved_GBps": gbs, "peak_GBps": PEAK_HBM_GBS, "frac": gbs / PEAK_HBM_GBS},

@@ -1,0 +1,76 @@
+"""Thread-local operator descriptor: the fields of the reference's ContextForDiffusionLM
+(prefilling_dllm/utils/context.py:8-24, 58-98, 126-155) that the attention operators consume.
+
+The reference assembles a dense block-diagonal boolean mask in __post_init__ (context.py:69-98).
+Here the mask stays a per-sequence description (`mask_kind` "full" / "causal", or a dense tensor
+in `block_mask` when the caller really has one), because the HIP kernels take the mask mode and
+read a dense mask only when one is given."""
+from __future__ import annotations
+
+import threading
+from dataclasses import dataclass
+from typing import Any, List, Optional
+
+import torch
+
+_THREAD_CONTEXT = threading.local()
+
+
+@dataclass
+class ContextForDiffusionLM:
+    is_prefill: bool = False
+    cu_seqlens_q: Optional[torch.Tensor] = None
+    cu_seqlens_k: Optional[torch.Tensor] = None
+    max_seqlen_q: int = 0
+    max_seqlen_k: int = 0
+    slot_mapping: Optional[torch.Tensor] = None
+    context_lens: Optional[torch.Tensor] = None
+    block_tables: Optional[torch.Tensor] = None
+    seqs: Optional[List[Any]] = None
+    seq_lens: Optional[List[int]] = None
+    seq_lens_ts: Optional[torch.Tensor] = None
+    kv_cache_layout: str = "unified"
+    need_kv_cache_store: bool = True
+    block_mask: Optional[torch.Tensor] = None      # dense [Nq, Nq] over the active rows, or None
+    decode_delta_state: Any = None
+    prefill_sparse_state: Any = None
+    mask_kind: str = "full"                        # "full" | "causal" | "dense"
+    # visible prefix as token ranges (range_ptr, range_start, range_len, max_ranges); None = the
+    # first context_lens[r] tokens of each page table (the reference's decode context)
+    ranges: Any = None
+    max_context_len: int = 0
+
+    def __post_init__(self):
+        if self.seq_lens_ts is not None and self.context_lens is not None:
+            self.total_lens = self.seq_lens_ts + self.context_lens
+        if self.block_mask is not None:
+            self.mask_kind = "dense"
+
+    @property
+    def total_num_seqs(self) -> int:
+        return len(self.seqs) if self.seqs is not None else 0
+
+
+def get_context_diffusion_lm() -> ContextForDiffusionLM:
+    ctx = getattr(_THREAD_CONTEXT, "diffusion_lm", None)
+    if ctx is None:
+        ctx = ContextForDiffusionLM()
+        _THREAD_CONTEXT.diffusion_lm = ctx
+    return ctx
+
+
+def set_context_diffusion_lm(is_prefill, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=0, max_seqlen_k=0,
+                             slot_mapping=None, context_lens=None, block_tables=None, seqs=None, seq_lens=None,
+                             seq_lens_ts=None, kv_cache_layout="unified", need_kv_cache_store=True,
+                             decode_delta_state=None, prefill_sparse_state=None, block_mask=None, mask_kind="full",
+                             ranges=None, max_context_len=0) -> None:
+    """Same positional/keyword surface as the reference (context.py:135-152) plus the mask / range
+    description the HIP path uses instead of a materialised mask."""
+    _THREAD_CONTEXT.diffusion_lm = ContextForDiffusionLM(
+        is_prefill, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, slot_mapping, context_lens, block_tables,
+        seqs, seq_lens, seq_lens_ts, kv_cache_layout, need_kv_cache_store, block_mask, decode_delta_state,
+        prefill_sparse_state, mask_kind, ranges, max_context_len)
+
+
+def reset_context_diffusion_lm() -> None:
+    _THREAD_CONTEXT.diffusion_lm = ContextForDiffusionLM()

@@ -1,0 +1,133 @@
+"""CPU-only checks: the C-ABI library loads and exports every symbol include/pdllm.h declares, error
+codes map to the reference's exception classes, and the host-side mirrors (allocator, record types)
+behave like the reference.  No kernel is launched here."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pdllm.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pdllm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from prefilling_dllm_amd import _lib
+    names = declared_symbols()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(_lib.lib, n), f"{n} declared in pdllm.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert _lib.lib.pdllm_abi_version() == 1
+    assert _lib.lib.pdllm_status_string(0) == b"ok"
+
+
+def test_header_compiles_as_c():
+    """The boundary is a plain C header: no C++ or HIP types in the signatures."""
+    src = '#include "pdllm.h"\nint main(void){ pdllm_attn_desc d; (void)d; return PDLLM_OK; }\n'
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-I", os.path.dirname(HEADER), "-x", "c",
+                        "-"], input=src.encode(), capture_output=True)
+    assert r.returncode == 0, r.stderr.decode()
+
+
+def test_struct_mirror_matches_header_layout():
+    """sizeof(pdllm_attn_desc) as the C compiler sees it == the ctypes mirror."""
+    from prefilling_dllm_amd import _lib
+    src = '#include <stdio.h>\n#include "pdllm.h"\nint main(void){ printf("%zu %zu %zu", sizeof(pdllm_attn_desc), ' \
+          '__builtin_offsetof(pdllm_attn_desc, q_stride), __builtin_offsetof(pdllm_attn_desc, sm_scale)); return 0; }\n'
+    exe = "/tmp/pdllm_sizeof"
+    r = subprocess.run(["gcc", "-I", os.path.dirname(HEADER), "-x", "c", "-", "-o", exe], input=src.encode(),
+                       capture_output=True)
+    assert r.returncode == 0, r.stderr.decode()
+    size, off_q, off_s = map(int, subprocess.check_output([exe]).split())
+    assert ctypes.sizeof(_lib.AttnDesc) == size
+    assert _lib.AttnDesc.q_stride.offset == off_q and _lib.AttnDesc.sm_scale.offset == off_s
+
+
+def test_status_codes_map_to_reference_exception_classes():
+    from prefilling_dllm_amd import _lib
+    _lib.check(0, "x")
+    for code, exc in ((-1, ValueError), (-2, ValueError), (-3, ValueError), (-5, RuntimeError), (-7, NotImplementedError)):
+        with pytest.raises(exc):
+            _lib.check(code, "x")
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    """Validation happens on the host before any launch: NULL pointers and bad shapes return codes."""
+    from prefilling_dllm_amd import _lib
+    lib = _lib.lib
+    assert lib.pdllm_kv_store(None, None, None, None, None, 1, 512, 512, 512, 10, None) == -1
+    assert lib.pdllm_topk_lowest_index(None, 1, 4, 4, 2, 1, None, None) == -1
+    assert lib.pdllm_attn_workspace_bytes(None) == -1
+    d = _lib.AttnDesc()
+    assert lib.pdllm_sparse_decode_attn(ctypes.byref(d), None) == -1
+    buf = (ctypes.c_char * 64)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    d.q = d.k_new = d.v_new = d.out = d.q_start_loc = p
+    d.head_dim, d.num_q_heads, d.num_kv_heads = 64, 4, 4
+    assert lib.pdllm_sparse_decode_attn(ctypes.byref(d), None) == -7            # head_dim != 128
+    d.head_dim, d.num_q_heads, d.num_kv_heads = 128, 6, 4
+    assert lib.pdllm_sparse_decode_attn(ctypes.byref(d), None) == -2            # heads not divisible
+    assert lib.pdllm_selfinfo_logprob(p, 10, p, 1, 100, p, 1 << 20, p, None) == -2   # stride < vocab
+    assert lib.pdllm_vocab_workspace_bytes(128, 152064) > 0
+
+
+def test_attention_plan_is_host_only():
+    from prefilling_dllm_amd import ops
+    rows, splits = ops.attention_plan(8, 28, 4, max_q_len=160, max_ctx_len=4096)
+    assert rows in (32, 64, 128, 160, 192) and splits >= 1
+    rows, splits = ops.attention_plan(1, 28, 4, max_q_len=32, max_ctx_len=32768)
+    assert splits > 1                                                            # few rows, long prefix: split KV
+    assert ops.attention_plan(8, 28, 4, max_q_len=160, max_ctx_len=4096, rows_per_group=128, num_splits=2) == (128, 2)
+
+
+def test_prefix_page_allocator_semantics():
+    """fastdllm_engine.py:88-167: free-list order, refcounts, exhaustion error, hash-keyed prefix reuse."""
+    from prefilling_dllm_amd.engine_ops import PrefixPageAllocator
+    import torch
+    a = PrefixPageAllocator(4, 256)
+    p = a.allocate_pages(3)
+    assert p == [0, 1, 2] and a.num_free_pages == 1
+    with pytest.raises(RuntimeError, match="Cannot allocate 2 pages, only 1 free"):
+        a.allocate_pages(2)
+    a.ref_pages([1])
+    a.release_pages([0, 1])
+    assert a.num_free_pages == 2 and a.page_ref_count[1] == 1        # page 1 still referenced
+    a.release_pages([1])
+    assert list(a.free_pages) == [3, 0, 1]
+    ids = [5, 6, 7]
+    e = a.register_prefix(ids, [2], 3, torch.zeros(4))
+    assert a.lookup_prefix(ids) is e and a.lookup_prefix([5, 6]) is None
+    assert a.compute_prompt_hash(ids) == a.compute_prompt_hash(list(ids))
+    e.ref_count = 1
+    assert not a.evict_one()
+    a.release_prefix(ids)
+    assert a.evict_one() and a.lookup_prefix(ids) is None and a.num_free_pages == 4
+
+
+def test_record_types_keep_the_reference_fields():
+    from prefilling_dllm_amd import engine_ops as e
+    import dataclasses
+    assert [f.name for f in dataclasses.fields(e.DreamPrefillRecord)] == [
+        "prompt_ids", "prompt_positions", "suffix_positions", "prompt_len", "full_prompt_len", "decode_len",
+        "prompt_page_ids", "block_page_ids", "first_token_id", "last_context_logit", "decode_delta_state",
+        "owns_prompt_pages", "cached_prefix", "kv_mode"]
+    assert [f.name for f in dataclasses.fields(e.DreamKVSnapshot)] == [
+        "prompt_len", "page_size", "kv_mode", "k_by_layer", "v_by_layer", "last_context_logit"]
+    assert [f.name for f in dataclasses.fields(e.FastDLLMEngineOutput)] == ["text", "token_ids", "n_diff_steps"]
+
+
+def test_product_path_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "prefilling-dllm_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.replace("# oracle", ""), f"{f} mentions the oracle"

@@ -254,3 +254,49 @@ def test_error_codes(dev):
     with pytest.raises(ValueError):
         ops.sparse_decode_attention(q.cpu(), k.cpu(), k.cpu(), None, None, None,
                                     torch.tensor([0, 32], dtype=torch.int32), max_q_len=32, max_ctx_len=0)
+
+
+def test_attention_layer_interface(dev):
+    """The layer mirror of attention_v4.Attention: a prefill that stores K/V into pages, then a decode
+    step of a 32-token block against that paged context, both checked against the oracle."""
+    from prefilling_dllm_amd.attention import Attention
+    from prefilling_dllm_amd.context import set_context_diffusion_lm, reset_context_diffusion_lm
+    gen = torch.Generator().manual_seed(31)
+    Hq, Hkv, d, P = 28, 4, 128, 256
+    prompt, block = 300, 32
+    scale = d ** -0.5
+    layer = Attention(Hq, d, scale, Hkv, "diffusion_lm")
+    layer.k_cache = torch.zeros(6, P, Hkv, d, dtype=torch.bfloat16, device=dev)
+    layer.v_cache = torch.zeros_like(layer.k_cache)
+    prompt_pages, block_pages = [4, 1], [3]
+    mk = lambda n, h: (torch.randn(n, h * d, generator=gen) / 3).to(torch.bfloat16)
+    q, k, v = mk(prompt + block, Hq), mk(prompt + block, Hkv), mk(prompt + block, Hkv)
+    slots = ref_ops.split_slot_mapping(prompt_pages, block_pages, prompt, block)
+    cu = torch.tensor([0, prompt + block], dtype=torch.int32, device=dev)
+    set_context_diffusion_lm(True, cu_seqlens_q=cu, cu_seqlens_k=cu, max_seqlen_q=prompt + block,
+                             max_seqlen_k=prompt + block, slot_mapping=slots.to(dev), mask_kind="full")
+    try:
+        o = layer(q.to(dev), k.to(dev), v.to(dev))
+    finally:
+        reset_context_diffusion_lm()
+    ref = ref_ops.chunk_prefill_attention(q.view(-1, Hq, d), k.view(-1, Hkv, d), v.view(-1, Hkv, d),
+                                          [0, prompt + block], causal=False, sm_scale=scale)
+    check(o.view(-1, Hq, d).float().cpu(), ref, tol=3e-2)
+    # decode step: replace the block, context = the prompt tokens in pages [4, 1]
+    q2, k2, v2 = mk(block, Hq), mk(block, Hkv), mk(block, Hkv)
+    slots2 = ref_ops.slot_mapping(block_pages, block)
+    cu2 = torch.tensor([0, block], dtype=torch.int32, device=dev)
+    bt = torch.tensor([prompt_pages + block_pages], dtype=torch.int32, device=dev)
+    set_context_diffusion_lm(False, cu_seqlens_q=cu2, max_seqlen_q=block, max_seqlen_k=prompt + block,
+                             slot_mapping=slots2.to(dev), context_lens=torch.tensor([prompt], dtype=torch.int32, device=dev),
+                             block_tables=bt, mask_kind="full")
+    try:
+        o2 = layer(q2.to(dev), k2.to(dev), v2.to(dev))
+    finally:
+        reset_context_diffusion_lm()
+    kc, vc = layer.k_cache.cpu(), layer.v_cache.cpu()
+    ref2 = ref_ops.sparse_decode_attention(q2.view(-1, Hq, d), k2.view(-1, Hkv, d), v2.view(-1, Hkv, d), kc, vc,
+                                           bt.cpu(), [0, block], [[(0, prompt)]], sm_scale=scale)
+    check(o2.view(-1, Hq, d).float().cpu(), ref2, tol=3e-2)
+    # the decode step stored the new block rows behind the prompt pages
+    assert torch.equal(kc[3, :block], k2.view(-1, Hkv, d))
