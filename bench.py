@@ -71,28 +71,36 @@ def algorithmic_work(q_len, ctx, n_req):
     return by, fl
 
 
-def prepare(ops, w, rows_per_group=0, num_splits=0):
+def prepare(ops, w, rows_per_group=0, num_splits=0, tiles_per_workgroup=0):
+    """One prepared descriptor per layer.  All layers of a step read the same page table and chunk
+    ranges, so they share one slot table, which every step rebuilds once (inside the timed region)."""
+    table = ops.new_slot_table(w["n_req"], w["ctx"], w["q"].device)
     preps = []
     for l in range(w["layers"]):
         preps.append(ops.PreparedAttention(w["q"][l], w["kn"][l], w["vn"][l], w["kv"][0, l], w["kv"][1, l],
                                            w["block_table"], w["qsl"], max_q_len=w["q_len"], max_ctx_len=w["ctx"],
                                            ranges=w["ranges"], out=w["out"][l], rows_per_group=rows_per_group,
-                                           num_splits=num_splits))
+                                           num_splits=num_splits, slot_table=table,
+                                           tiles_per_workgroup=tiles_per_workgroup))
     return preps
+
+
+def run_step(preps, stream):
+    preps[0].build_slot_table(stream)
+    for p in preps:
+        p.run(stream)
 
 
 def time_steps(torch, preps, steps, warmup):
     stream = torch.cuda.current_stream().cuda_stream
     for _ in range(warmup):
-        for p in preps:
-            p.run(stream)
+        run_step(preps, stream)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
     for _ in range(steps):
-        for p in preps:
-            p.run(stream)
+        run_step(preps, stream)
     e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -127,6 +135,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--rows-per-group", type=int, default=0, help="override the row-group size (tuning)")
     ap.add_argument("--num-splits", type=int, default=0, help="override the KV split count (tuning)")
+    ap.add_argument("--tiles-per-wg", type=int, default=0, help="override the tiles per workgroup (tuning)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
@@ -156,7 +165,7 @@ def main():
         del src, dst
 
     w = build_workload(torch, dev)
-    preps = prepare(ops, w, args.rows_per_group, args.num_splits)
+    preps = prepare(ops, w, args.rows_per_group, args.num_splits, args.tiles_per_wg)
     wall, gpu_s = time_steps(torch, preps, args.steps, args.warmup)
     launches = args.steps * w["layers"]
     us_per_step = gpu_s / args.steps * 1e6
@@ -202,7 +211,7 @@ def main():
                    "rows_per_workgroup": rows, "kv_splits": splits},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(w["q_len"]) if not (args.rows_per_group or args.num_splits) else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(w["q_len"]) if not (args.rows_per_group or args.num_splits or args.tiles_per_wg) else None,
                      "kernel": "attn_fwd_kernel", "avg_launch_us": launch_s * 1e6,
                      "algorithmic_flops_per_launch": fl, "algorithmic_bytes_per_launch": by},
         "hbm": {"achieved_GBps": gbs, "peak_GBps": PEAK_HBM_GBS, "frac": gbs / PEAK_HBM_GBS},

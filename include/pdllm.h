@@ -120,19 +120,29 @@ typedef struct pdllm_attn_desc {
   int32_t scale_page_stride, scale_head_stride;
   int32_t n_req;
   int32_t max_q_len;   /* host upper bound of the per-request active length   */
-  int32_t max_ctx_len; /* host upper bound of the per-request visible prefix  */
+  int32_t max_ctx_len; /* host upper bound of the per-request visible prefix; keys beyond it are not seen */
   int32_t max_ranges;  /* host upper bound of ranges per request (<= 128)     */
   int32_t num_q_heads, num_kv_heads, head_dim; /* head_dim must be 128        */
   int32_t page_size;   /* power of two                                        */
   int32_t kv_dtype;    /* PDLLM_KV_*  (dtype of the cache; in-flight K/V are bf16) */
   int32_t mask_mode;   /* PDLLM_MASK_*                                        */
-  int32_t num_splits;  /* 0 = choose; >0 = force this many KV splits          */
+  int32_t num_splits;  /* 0 = choose; 1..16 = cut every column into this many equal KV splits */
   int32_t rows_per_group; /* 0 = choose; else 32*J, J in {1,2,4,5,6,8}        */
   float sm_scale;      /* softmax scale (1/sqrt(d) when the caller has no own) */
+  /* optional: the slot table of the visible prefix, built by pdllm_attn_build_slot_table from
+   * block_table and the ranges.  It only depends on those, so one table serves every layer of
+   * a step.  NULL = pdllm_sparse_decode_attn builds it in the workspace on every call. */
+  const int32_t* slot_table;
+  int64_t slot_table_stride; /* int32 entries per request, >= pdllm_attn_slot_table_stride() */
+  /* 0 = choose; >0 = every workgroup takes this many consecutive 64-key tiles of the line formed
+   * by the tiles of all (request, KV head, row group) columns, so a workgroup may finish one column
+   * and start the next; columns cut into pieces are merged from fp32 partials in the workspace.
+   * Overrides num_splits. */
+  int32_t tiles_per_workgroup;
 } pdllm_attn_desc;
 
-/* Bytes of workspace pdllm_sparse_decode_attn needs for this descriptor
- * (0 when no KV split is used).  Negative = error code. */
+/* Bytes of workspace pdllm_sparse_decode_attn needs for this descriptor: split-KV partials
+ * and, when desc->slot_table is NULL, the slot table.  Negative = error code. */
 int64_t pdllm_attn_workspace_bytes(const pdllm_attn_desc* desc);
 
 /* Replaces the decode branch of Attention.forward (layers/attention/attention_v4.py:368-397),
@@ -152,6 +162,17 @@ int pdllm_sparse_decode_attn(const pdllm_attn_desc* desc, pdllm_stream_t stream)
  * in-flight tensors, q_start_loc (= cu_seqlens), mask_mode and cache fields. */
 int pdllm_chunk_prefill_attn(const pdllm_attn_desc* desc, const int32_t* slot_mapping,
                              pdllm_stream_t stream);
+
+/* Replaces the per-forward context arrays of the reference (slot_mapping / block_tables of
+ * ContextForDiffusionLM, utils/context.py:58-67, built once per step for all layers; slot
+ * formula ENG:331-337): table[r*table_stride + v] = page*page_size + offset of the v-th visible
+ * prefix key of request r (the ranges in order, through block_table[r]); entries up to the next
+ * multiple of 64 repeat a valid slot; table[r*table_stride + table_stride-1] = number of
+ * visible keys = min(sum of range lengths, max_ctx_len).  Uses block_table, bt_stride, range_*,
+ * max_ranges, n_req, max_ctx_len, page_size and n_pages of the descriptor. */
+int64_t pdllm_attn_slot_table_stride(const pdllm_attn_desc* desc);
+int pdllm_attn_build_slot_table(const pdllm_attn_desc* desc, int32_t* table, int64_t table_stride,
+                                pdllm_stream_t stream);
 
 /* The plan pdllm_sparse_decode_attn (prefill == 0) or pdllm_chunk_prefill_attn would use:
  * rows per workgroup (32 * row blocks) and number of KV splits.  For tuning and tests. */

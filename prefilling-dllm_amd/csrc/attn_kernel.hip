@@ -11,26 +11,28 @@
 //   A row group is J blocks of 32 "rows"; a row is one (query token, q-head of the GQA
 //   group) pair, ordered token-major, so all G q-heads of a KV head reuse every K/V tile.
 //   With J >= 4 wave w owns row block w ("slot A") for all keys.  The remaining blocks
-//   ("slot B") are split over waves INSIDE every 128-key tile, so that all waves do the same
-//   amount of MFMA work per tile: J=5 -> block 4, wave w takes key block w of each tile;
-//   J=6 -> blocks 4,5, two key blocks per wave; J=8 -> a second full block per wave.
-//   J=1,2 have only shared blocks (intra-workgroup split-KV for short active blocks).
-//   Slot B issues its MFMAs on the operand fragments slot A has just read, so it adds no
-//   LDS traffic; shared blocks are merged through LDS with a log-sum-exp reduction.
-//   An optional split over workgroups writes fp32 partials + LSE to a workspace that
-//   attn_merge_kernel reduces.
+//   ("slot B") are shared: J=6 -> blocks 4,5, each split between two waves that take one
+//   32-key block of every tile; J=5 -> block 4 split over all four waves, two of them on even
+//   tiles and two on odd tiles; J=8 -> a second full block per wave.  J=1,2 have only shared
+//   blocks (intra-workgroup split-KV for short active blocks).  Shared blocks are merged
+//   through LDS with a log-sum-exp reduction.  An optional split over workgroups writes fp32
+//   partials + LSE to a workspace that attn_merge_kernel reduces.
+//   The tile buffers take 64 KB of LDS and a wave at most 256 registers, so two workgroups
+//   share a CU: while one waits for the matrix unit the other runs its softmax.
 //
-// Per 128-key tile
+// Per 64-key tile
 //   K and V rows are copied HBM -> LDS by global_load_lds (16 bytes per lane, no registers);
-//   the row addresses come from a slot table that 128 threads resolve through the page table
+//   the row addresses come from a slot table that 64 threads resolve through the page table
 //   two tiles ahead.  Rows are 256 bytes = 16 chunks; chunk c of row r is stored at position
 //   c ^ rotl4(r & 15), which makes the 128-bit K operand reads and the transposing
 //   ds_read_b64_tr_b16 V operand reads bank-conflict free.
 //   S^T = K Q^T and O^T += V^T P^T use v_mfma_f32_32x32x16_bf16; in the S^T accumulator
 //   layout a lane holds 16 keys of one query, so softmax statistics are lane-local plus
-//   one half-wave exchange, and P^T feeds the second MFMA straight from registers.  The
-//   running maximum is only advanced (and O rescaled) when a tile exceeds it by more than
-//   2^8, which removes most rescale work without changing the result.
+//   one half-wave exchange, and P^T feeds the second MFMA straight from registers.
+//   Q is multiplied by sm_scale * log2(e) once, and the S^T accumulators start at minus the
+//   running maximum, so the MFMA result is the exponent itself.  The running maximum is only
+//   advanced (and O rescaled) when a tile exceeds it by more than 2^8, which removes most
+//   rescale work without changing the result.
 //   fp8 e4m3 pages are dequantised (x * scale[page]) in registers while staging.
 
 #include <type_traits>
@@ -47,18 +49,20 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
 constexpr int kD = 128;          // head dim
-constexpr int kKT = 128;         // keys per tile
+constexpr int kKT = 64;          // keys per tile
+constexpr int kNKB = kKT / 32;   // 32-key blocks per tile
 constexpr int kThreads = 256;    // 4 wavefronts
 constexpr int kRowBytes = 256;   // one K or V row in LDS
-constexpr int kTileBytes = kKT * kRowBytes;      // 32768
+constexpr int kTileBytes = kKT * kRowBytes;      // 16384
 constexpr int kBufBytes = 2 * kTileBytes;        // K tile + V tile
-constexpr int kMainBytes = 2 * kBufBytes;        // double buffered: 131072
-constexpr int kPartStride = 33;                  // floats per d-row of an LDS partial
-constexpr int kPartBytes = kD * kPartStride * 4; // 16896
+constexpr int kMainBytes = 2 * kBufBytes;        // double buffered: 65536
+constexpr int kDmaGroups = kKT / 16;             // 16-row groups of a tile; a wave copies 4 rows of each
+constexpr int kPartBytes = kD * 32 * 4;          // LDS partial of a shared row block: [d][row ^ (d & 31)] fp32
 constexpr int kMaxRanges = 128;
 constexpr int kMaxTok = 264;                     // query tokens a row group of 256 rows can touch (+ slack)
 constexpr float kRescaleSlack = 8.f;             // log2 units
 static_assert(4 * kPartBytes <= kMainBytes, "partials must fit the tile buffers");
+static_assert(kNKB == 2, "the shared-block schedule assumes two key blocks per tile");
 
 struct AttnKParams {
   const __bf16* q;
@@ -74,6 +78,8 @@ struct AttnKParams {
   const int* range_ptr;
   const int* range_start;
   const int* range_len;
+  const int* slot_table;  // [n_req, slot_stride]: cache slot of every visible prefix key; last entry = key count
+  long slot_stride;
   const uint8_t* mask;
   float* ws_o;
   float* ws_lse;
@@ -86,10 +92,17 @@ struct AttnKParams {
   int scale_page_stride, scale_head_stride;
   int n_req, Hq, Hkv, G;
   int page_shift;
+  int max_ctx_len;
+  int max_ranges;
   int mask_mode;
   int J;
   int row_tiles;
-  int num_splits;
+  // work decomposition: the tiles of all columns (request, KV head, row group) form one line of
+  // n_cols * t_lin positions that is cut into spans of `span` tiles, one per workgroup
+  int t_lin;       // positions per column (>= the largest tile count of a column)
+  int span;        // tiles per workgroup
+  int n_lin;       // n_cols * t_lin
+  int max_pieces;  // partial results per row in the workspace
   int max_q_len;
   float scale_log2;  // sm_scale * log2(e)
 };
@@ -127,13 +140,38 @@ __device__ __forceinline__ uint4 dequant_fp8x8(uint32_t lo, uint32_t hi, float s
   return r;
 }
 
-// Softmax update of one row block over NKB key blocks of 32 keys (S holds raw scores in the
-// S^T accumulator layout: element i of a lane is key 8*(i/4) + 4*h + i%4 of the block).
+// LDS operand reads of the MFMA loops are issued and awaited by hand.  The compiler would make
+// every LDS read wait for the direct-to-LDS copies of the next tile that are in flight (it
+// cannot tell that they go to the other buffer), which serialises copy and compute.  The asm
+// reads are invisible to its wait-count bookkeeping, so each consumer waits explicitly:
+// lds_wait<N>(x) blocks until at most N younger LDS operations are outstanding and ties the
+// wait to the registers x that the operation filled.
+template <int OFF>
+__device__ __forceinline__ void lds_read_b128(bf16x8& dst, unsigned addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int OFF>
+__device__ __forceinline__ void lds_read_tr16_b64(s16x4& dst, unsigned addr) {
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int N, typename T>
+__device__ __forceinline__ void lds_wait(T& x) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N) : "memory");
+}
+template <int N, typename T>
+__device__ __forceinline__ void lds_wait2(T& x, T& y) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N) : "memory");
+}
+
+// Softmax update of one row block over NKB key blocks of 32 keys.  S holds the exponents in
+// log2 units relative to the running maximum M (the accumulators were started at -M, or at 0
+// while M is still -inf), in the S^T accumulator layout: element i of a lane is key
+// 8*(i/4) + 4*h + i%4 of the block.
 // generic (wave-uniform): keys >= lim_tile (per lane: tile bound and causal bound) and keys whose
 // bit in mrow[key block] is clear are masked out.
 template <int NKB>
 __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB][2], f32x16 (&O)[4],
-                                               float& M, float& l, float c, int h, int kb_first, bool generic,
+                                               float& M, float& l, int h, int kb_first, bool generic,
                                                int lim_tile, const uint32_t* mrow) {
   if (generic) {
 #pragma unroll
@@ -150,19 +188,25 @@ __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB
       }
     }
   }
-  float mx = S[0][0];
+  float mx = fmaxf(S[0][0], S[0][1]);
 #pragma unroll
   for (int b = 0; b < NKB; ++b)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, S[b][i]);
-  mx = half_swap_max(mx) * c;  // scaled to log2 units (c > 0)
+    for (int i = (b == 0 ? 2 : 0); i < 16; i += 2) mx = fmaxf(fmaxf(mx, S[b][i]), S[b][i + 1]);
+  mx = half_swap_max(mx);
   // advance the reference maximum only when some row of the wave needs it
-  const bool need = mx > M + kRescaleSlack || (M == -INFINITY && mx > -INFINITY);
+  const bool need = mx > kRescaleSlack || (M == -INFINITY && mx > -INFINITY);
   if (__builtin_amdgcn_ballot_w64(need) != 0) {
-    const float Mn = fmaxf(M, mx);
+    const float Muse = (M == -INFINITY) ? 0.f : M;
+    const float Mn = fmaxf(M, Muse + mx);  // mx = -inf (nothing visible) keeps M
     const float alpha = (Mn == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(M - Mn);  // M = -inf -> 0
+    const float delta = ((Mn == -INFINITY) ? 0.f : Mn) - Muse;
     M = Mn;
     l *= alpha;
+#pragma unroll
+    for (int b = 0; b < NKB; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) S[b][i] -= delta;
 #pragma unroll
     for (int db = 0; db < 4; ++db) {
 #pragma unroll
@@ -170,40 +214,41 @@ __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB
       __builtin_amdgcn_sched_barrier(0);  // one accumulator block at a time through the VALU registers
     }
   }
-  const float Muse = (M == -INFINITY) ? 0.f : M;
+  // p = 2^S rounded to bf16; the row sum is taken over the rounded values, the same ones the
+  // second MFMA multiplies with V
+  const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
   float psum = 0.f;
 #pragma unroll
   for (int b = 0; b < NKB; ++b) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(S[b][i], c, -Muse));
-      S[b][i] = pv;
-      psum += pv;
-    }
-#pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) P[b][j][e] = (__bf16)S[b][8 * j + e];
+      for (int e = 0; e < 8; e += 2) {
+        const bf16x2 pr = {(__bf16)__builtin_amdgcn_exp2f(S[b][8 * j + e]),
+                           (__bf16)__builtin_amdgcn_exp2f(S[b][8 * j + e + 1])};
+        psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);
+        P[b][j][e] = pr[0];
+        P[b][j][e + 1] = pr[1];
+      }
   }
   l += psum;
 }
 
 template <int KV_FP8, int J>
-__global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p) {
+__global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd_kernel(const AttnKParams p) {
   constexpr bool HAS_A = J >= 4;
-  constexpr int NB = (J == 1 || J == 5) ? 1 : (J == 2 || J == 6) ? 2 : (J == 8) ? 4 : 0;
-  constexpr int NBA = NB > 0 ? NB : 1;  // array extents must be positive
+  constexpr bool DUAL = J == 8;                                  // slot B = a second full block per wave
+  constexpr bool HAS_B = J != 4;
   constexpr int GS = (J == 1 || J == 5) ? 4 : (J == 2 || J == 6) ? 2 : 1;  // waves sharing a B block
+  constexpr bool QB_LDS = J == 5 || J == 6;  // Q of the shared block(s) lives in LDS, not in registers
 
   __shared__ __attribute__((aligned(1024))) char lds[kMainBytes];
   __shared__ float s_ml[4][2][32];
-  __shared__ int s_cum[kMaxRanges + 1];
-  __shared__ int s_start[kMaxRanges];
-  __shared__ int s_len[kMaxRanges];
-  __shared__ unsigned s_koff[3][kKT];  // row offsets of a tile's keys in 16-byte units (K and V source)
-  __shared__ unsigned s_voff[3][kKT];
-  __shared__ int s_page[KV_FP8 ? 3 : 1][KV_FP8 ? kKT : 1];  // fp8: page of each key (scale lookup)
-  __shared__ uint32_t s_maskbits[2][kMaxTok][4];  // dense mask of an active tile, one bit per key
+  // dynamic part: Q fragments of the shared blocks (QB_LDS), then the dense-mask bit rows
+  // [2][kMaxTok][kNKB] of an active tile (one bit per key; only with PDLLM_MASK_DENSE)
+  extern __shared__ __attribute__((aligned(16))) char dyn_lds[];
+  constexpr int kQbBytes = QB_LDS ? (J - 4) * 8192 : 0;
+  uint32_t (*s_maskbits)[kMaxTok][kNKB] = reinterpret_cast<uint32_t (*)[kMaxTok][kNKB]>(dyn_lds + kQbBytes);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -211,99 +256,11 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
   const int l32 = lane & 31;
   const int h = lane >> 5;
 
-  int lid = xcd_remap(blockIdx.x, gridDim.x);
-  const int row_tile = lid % p.row_tiles;
-  lid /= p.row_tiles;
-  const int split = lid % p.num_splits;
-  lid /= p.num_splits;
-  const int kvh = lid % p.Hkv;
-  const int req = lid / p.Hkv;
-
   const int G = p.G;
-  const int q0 = p.q_start_loc[req];
-  const int Sq = p.q_start_loc[req + 1] - q0;
-  if (q0 < 0 || Sq <= 0 || (long)q0 + Sq > p.n_tokens || Sq > p.max_q_len) return;
-  const int rows = Sq * G;
-  const int row0 = row_tile * 32 * J;
-  if (row0 >= rows) return;
+  const float c = p.scale_log2;
+  const unsigned lds_base = (unsigned)(size_t)lds;  // LDS address of the tile buffers
 
-  // ---- visible prefix ranges of this request -> cumulative key counts in LDS ----
-  int nr = 0;
-  if (p.k_cache != nullptr && p.range_ptr != nullptr) {
-    const int r0 = p.range_ptr[req];
-    nr = p.range_ptr[req + 1] - r0;
-    nr = nr < 0 ? 0 : (nr > kMaxRanges ? kMaxRanges : nr);
-    if (tid < nr) {
-      const int len = p.range_len[r0 + tid];
-      s_len[tid] = len > 0 ? len : 0;
-      s_start[tid] = p.range_start[r0 + tid];
-    }
-  }
-  __syncthreads();
-  if (tid <= nr) {
-    int cc = 0;
-    for (int i = 0; i < tid; ++i) cc += s_len[i];
-    s_cum[tid] = cc;
-  }
-  __syncthreads();
-  const int ctx_total = s_cum[nr];
-
-  const int Tc = (ctx_total + kKT - 1) / kKT;
-  int Sa = Sq;
-  if (p.mask_mode == PDLLM_MASK_CAUSAL) {
-    const int last_row = (row0 + 32 * J < rows ? row0 + 32 * J : rows) - 1;
-    const int lim = last_row / G + 1;
-    Sa = lim < Sq ? lim : Sq;
-  }
-  const int Ta = (Sa + kKT - 1) / kKT;
-  const int T = Tc + Ta;
-  const int tps = (T + p.num_splits - 1) / p.num_splits;
-  const int T0 = split * tps < T ? split * tps : T;
-  const int T1 = T0 + tps < T ? T0 + tps : T;
-
-  // ---- row blocks of this wave ----
-  const int blkA = wave;
-  int blkB = -1, kb0 = 0, gi = 0;
-  if (J == 1) { blkB = 0; kb0 = wave; gi = wave; }
-  else if (J == 2) { blkB = wave >> 1; kb0 = 2 * (wave & 1); gi = wave & 1; }
-  else if (J == 5) { blkB = 4; kb0 = wave; gi = wave; }
-  else if (J == 6) { blkB = 4 + (wave >> 1); kb0 = 2 * (wave & 1); gi = wave & 1; }
-  else if (J == 8) { blkB = 4 + wave; }
-  const int bmask = ((1 << NB) - 1) << kb0;  // key blocks of a tile this wave handles for slot B
-
-  // ---- Q fragments (B operand of S^T = K Q^T), rows of this lane ----
-  bf16x8 QA[8], QB[8];
-  int srowA = 0, srowB = 0, ridxA = -1, ridxB = -1;
-  auto load_q = [&](int blk, bf16x8 (&Q)[8], int& srow, int& ridx) __attribute__((always_inline)) {
-    const int r = row0 + 32 * blk + l32;
-    const bool valid = blk >= 0 && r < rows;
-    const int rr = valid ? r : 0;
-    const int tq = rr / G;
-    const int g = rr - tq * G;
-    srow = tq;
-    ridx = valid ? r : -1;
-    const __bf16* qp = p.q + (long)(q0 + tq) * p.q_stride + (long)(kvh * G + g) * kD + 8 * h;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      if (valid) {
-        Q[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) Q[ks][e] = (__bf16)0.f;
-      }
-    }
-  };
-  if (HAS_A) load_q(blkA, QA, srowA, ridxA);
-  if (NB > 0) load_q(blkB, QB, srowB, ridxB);
-
-  f32x16 OA[4], OB[4];
-  float MA = -INFINITY, MB = -INFINITY, lA = 0.f, lB = 0.f;
-#pragma unroll
-  for (int db = 0; db < 4; ++db)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) { OA[db][i] = 0.f; OB[db][i] = 0.f; }
-
-  // ---- per-lane LDS operand offsets (bytes inside a tile) ----
+  // per-lane LDS operand offsets (bytes inside a tile)
   int koff[8];
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) koff[ks] = l32 * kRowBytes + (((2 * ks + h) ^ swz(l32)) << 4);
@@ -321,46 +278,107 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
     }
   }
 
-  // ---- slot table: logical key of a tile -> cache slot (or active row), resolved by 128 threads ----
-  // Two phases so that the page-table load is in flight while the tile is computed:
-  // resolve_begin finds the logical token and issues the load, resolve_end publishes the slot.
-  const int page_mask = (1 << p.page_shift) - 1;
-  int rp = 0;
-  int rs_page = 0, rs_low = 0;
-  auto resolve_begin = [&](int t) __attribute__((always_inline)) {
-    if (tid >= kKT) return;
-    if (t < Tc) {
-      int v = t * kKT + tid;
-      if (v >= ctx_total) v = t * kKT;  // padding rows copy the first (always valid) row; they are masked
-      if (v < s_cum[rp]) rp = 0;
-      while (v >= s_cum[rp + 1]) ++rp;
-      const int tok = s_start[rp] + (v - s_cum[rp]);
-      int pi = tok >> p.page_shift;
-      pi = pi < 0 ? 0 : (pi >= p.bt_stride ? p.bt_stride - 1 : pi);
-      rs_page = p.block_table[(long)req * p.bt_stride + pi];
-      rs_low = tok & page_mask;
-    } else {
-      const int a = (t - Tc) * kKT + tid;
-      rs_page = -1;
-      rs_low = a < Sa ? a : (t - Tc) * kKT;
+  // this workgroup's span of the tile line; it may cover the end of one column and the start of
+  // the next, each part ("piece") is an attention pass of its own
+  const int wg = xcd_remap(blockIdx.x, gridDim.x);
+  int x = wg * p.span;
+  const int x_end = x + p.span < p.n_lin ? x + p.span : p.n_lin;
+  while (x < x_end) {
+  const int col = x / p.t_lin;
+  const int tb = x - col * p.t_lin;
+  const int te = tb + (x_end - x) < p.t_lin ? tb + (x_end - x) : p.t_lin;
+  x += te - tb;
+  const int wg_first = (col * p.t_lin) / p.span;            // workgroups holding pieces of this column
+  const int wg_last = ((col + 1) * p.t_lin - 1) / p.span;
+  const int piece = wg - wg_first;
+  const bool whole = wg_first == wg_last;  // the only piece: write the result, not a partial
+  const int row_tile = col % p.row_tiles;
+  const int kvh = (col / p.row_tiles) % p.Hkv;
+  const int req = col / (p.row_tiles * p.Hkv);
+
+  const int q0 = p.q_start_loc[req];
+  const int Sq = p.q_start_loc[req + 1] - q0;
+  if (q0 < 0 || Sq <= 0 || (long)q0 + Sq > p.n_tokens || Sq > p.max_q_len) continue;
+  const int rows = Sq * G;
+  const int row0 = row_tile * 32 * J;
+  if (row0 >= rows) continue;
+  // lane coordinates for the prologue and epilogue of a piece, made opaque per piece so that the
+  // address arithmetic built on them is not hoisted out of the piece loop (it would stay live in
+  // registers through the tile loop)
+  int lane_e = lane;
+  asm volatile("" : "+v"(lane_e));
+  const int l32e = lane_e & 31;
+  const int he = lane_e >> 5;
+
+  // visible prefix keys of this request: count and slots come from the slot table
+  const int* tbl = p.slot_table != nullptr ? p.slot_table + (long)req * p.slot_stride : nullptr;
+  int ctx_total = tbl != nullptr ? tbl[p.slot_stride - 1] : 0;
+  ctx_total = __builtin_amdgcn_readfirstlane(ctx_total);
+  const int Tc = (ctx_total + kKT - 1) / kKT;
+  int Sa = Sq;
+  if (p.mask_mode == PDLLM_MASK_CAUSAL) {
+    const int last_row = (row0 + 32 * J < rows ? row0 + 32 * J : rows) - 1;
+    const int lim = last_row / G + 1;
+    Sa = lim < Sq ? lim : Sq;
+  }
+  const int Ta = (Sa + kKT - 1) / kKT;
+  const int T = Tc + Ta;
+  const int T0 = tb < T ? tb : T;
+  const int T1 = te < T ? te : T;
+
+  // ---- row blocks of this wave ----
+  const int blkA = wave;
+  const int gi = wave & (GS - 1);  // index of this wave among the GS waves sharing its B block
+  int blkB = -1;
+  if (J == 1) blkB = 0;
+  else if (J == 2) blkB = wave >> 1;
+  else if (J == 5) blkB = 4;
+  else if (J == 6) blkB = 4 + (wave >> 1);
+  else if (J == 8) blkB = 4 + wave;
+  const int kbB = gi & 1;       // key block of a tile this wave handles for a shared block
+  const int parB = (gi >> 1) ^ (row_tile & 1);  // GS == 4: tiles of this parity only
+
+  // ---- Q fragments (B operand of S^T = K Q^T), rows of this lane, scaled to log2 units ----
+  bf16x8 QA[8], QB[8];
+  int srowA = 0, srowB = 0, ridxA = -1, ridxB = -1;
+  auto load_q = [&](int blk, bf16x8 (&Q)[8], int& srow, int& ridx) __attribute__((always_inline)) {
+    const int r = row0 + 32 * blk + l32e;
+    const bool valid = blk >= 0 && r < rows;
+    const int rr = valid ? r : 0;
+    const int tq = rr / G;
+    const int g = rr - tq * G;
+    srow = tq;
+    ridx = valid ? r : -1;
+    const __bf16* qp = p.q + (long)(q0 + tq) * p.q_stride + (long)(kvh * G + g) * kD + 8 * he;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      if (valid) {
+        const bf16x8 raw = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) Q[ks][e] = (__bf16)((float)raw[e] * c);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) Q[ks][e] = (__bf16)0.f;
+      }
     }
   };
-  const long cache_row_bytes = p.cache_token_stride * (KV_FP8 ? 1 : 2);
-  auto resolve_end = [&](int t, int sb) __attribute__((always_inline)) {
-    if (tid >= kKT) return;
-    if (t < Tc) {
-      int page = rs_page;
-      page = page < 0 ? 0 : (page >= p.n_pages ? p.n_pages - 1 : page);  // never read out of bounds
-      const long slot = ((long)page << p.page_shift) + rs_low;
-      const unsigned off = (unsigned)((slot * cache_row_bytes) >> 4);
-      s_koff[sb][tid] = off;
-      s_voff[sb][tid] = off;
-      if (KV_FP8) s_page[sb][tid] = page;
-    } else {
-      s_koff[sb][tid] = (unsigned)(((long)rs_low * p.kn_stride * 2) >> 4);
-      s_voff[sb][tid] = (unsigned)(((long)rs_low * p.vn_stride * 2) >> 4);
-    }
-  };
+  if (HAS_A) load_q(blkA, QA, srowA, ridxA);
+  if (HAS_B) load_q(blkB, QB, srowB, ridxB);
+  // shared block with a slot A next to it: park its fragments in LDS as [block][ks][lane] x 16 B
+  // (every wave of the group holds the same values; the first one writes)
+  const int qb_off = QB_LDS ? (blkB - 4) * 8192 + lane * 16 : 0;
+  const int qb_off_e = QB_LDS ? (blkB - 4) * 8192 + lane_e * 16 : 0;
+  if (QB_LDS && gi == 0) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) *reinterpret_cast<bf16x8*>(dyn_lds + qb_off_e + ks * 1024) = QB[ks];
+  }
+
+  f32x16 OA[4], OB[4];
+  float MA = -INFINITY, MB = -INFINITY, lA = 0.f, lB = 0.f;
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { OA[db][i] = 0.f; OB[db][i] = 0.f; }
 
   // dense mask of active tile t -> bit rows in LDS (built one tile ahead, like the slot table)
   const uint8_t* mask_base = p.mask != nullptr ? p.mask + (long)q0 * p.mask_stride + q0 : nullptr;
@@ -370,8 +388,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
   auto build_mask = [&](int t, int par) __attribute__((always_inline)) {
     if (p.mask_mode != PDLLM_MASK_DENSE || t < Tc) return;
     const int a0 = (t - Tc) * kKT;
-    for (int idx = tid; idx < ntok * 4; idx += kThreads) {
-      const int tok = idx >> 2, w = idx & 3;
+    for (int idx = tid; idx < ntok * kNKB; idx += kThreads) {
+      const int tok = idx / kNKB, w = idx % kNKB;
       const uint8_t* mp = mask_base + (long)(tq_first + tok) * p.mask_stride + a0 + 32 * w;
       uint32_t bits = 0;
       for (int j = 0; j < 32; ++j)
@@ -381,11 +399,14 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
   };
 
   // fp8 staging registers (only used by the fp8 instantiations)
-  uint2 st_k[8], st_v[8];
-  float st_ks[8], st_vs[8];
+  uint2 st_k[kDmaGroups], st_v[kDmaGroups];
+  float st_ks[kDmaGroups], st_vs[kDmaGroups];
 
-  // issue the copy of tile t into buffer `buf`: rows 4*ii + lane/16 for ii = i*4 + wave.
-  // The chunk a lane fetches, (lane & 15) ^ swz(row), does not depend on i because 16 | 16*i.
+  // Copy of tile t into buffer `buf`: this wave moves rows 16*i + 4*wave + lane/16 for each 16-row
+  // group i, one instruction for K and one for V.  The chunk a lane fetches,
+  // (lane & 15) ^ swz(row), does not depend on i because the swizzle has period 16.
+  // The source rows are cache slots read from the slot table (prefix tiles) or rows of the
+  // active block; they are fetched into registers one tile before the copy is issued.
   const int lane_row = 4 * wave + (lane >> 4);
   const int lane_ch = (lane & 15) ^ swz(lane_row);
   const long cache_lane_off = ((long)kvh * p.cache_head_stride + 8 * lane_ch) * (KV_FP8 ? 1 : 2);
@@ -393,72 +414,59 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
   const char* vc_lane = static_cast<const char*>(p.v_cache) + cache_lane_off;
   const char* kn_lane = reinterpret_cast<const char*>(p.k_new + (long)q0 * p.kn_stride + kvh * kD + 8 * lane_ch);
   const char* vn_lane = reinterpret_cast<const char*>(p.v_new + (long)q0 * p.vn_stride + kvh * kD + 8 * lane_ch);
-  // Tile copy = 16 wave-level instructions (8 row groups x {K, V}).  They are handed out one at a
-  // time between the MFMAs of the tile before, so that the memory pipeline never blocks the wave.
-  unsigned dma_ko[8], dma_vo[8];
-  const char* dma_kb = nullptr;
-  const char* dma_vb = nullptr;
-  char* dma_dst = nullptr;
-  bool dma_on = false, dma_fp8 = false;
-  int dma_sb = 0;
-  auto dma_begin = [&](int t, int sb, int buf, bool on) __attribute__((always_inline)) {
-    dma_on = on;
-    const bool ctx = t < Tc;
-    dma_fp8 = KV_FP8 && ctx;
-    dma_sb = sb;
-    dma_kb = ctx ? kc_lane : kn_lane;
-    dma_vb = ctx ? vc_lane : vn_lane;
-    dma_dst = lds + buf * kBufBytes + wave * 1024;
-  };
-  // load the source offsets of row groups [I0, I1) from the slot table
-  auto dma_offsets = [&](auto i0_tag, auto i1_tag) __attribute__((always_inline)) {
-    constexpr int I0 = decltype(i0_tag)::value, I1 = decltype(i1_tag)::value;
-    if (!dma_on) return;
+  const unsigned cache_row16 = (unsigned)((p.cache_token_stride * (KV_FP8 ? 1 : 2)) >> 4);  // 16-byte units
+  const unsigned kn_row16 = (unsigned)((p.kn_stride * 2) >> 4);
+  const unsigned vn_row16 = (unsigned)((p.vn_stride * 2) >> 4);
+  int nslot[kDmaGroups];
+  auto load_slots = [&](int t) __attribute__((always_inline)) {
+    if (t < Tc) {
 #pragma unroll
-    for (int i = I0; i < I1; ++i) {
-      dma_ko[i] = s_koff[dma_sb][16 * i + lane_row];
-      dma_vo[i] = s_voff[dma_sb][16 * i + lane_row];
+      for (int i = 0; i < kDmaGroups; ++i) nslot[i] = tbl[t * kKT + 16 * i + lane_row];
+    } else {
+      const int a0 = (t - Tc) * kKT;
+#pragma unroll
+      for (int i = 0; i < kDmaGroups; ++i) {
+        const int a = a0 + 16 * i + lane_row;
+        nslot[i] = a < Sa ? a : a0;  // padding rows copy the first (always valid) row; they are masked
+      }
     }
   };
-  // issue instruction `k` of the tile copy: row group k / 2, K (even k) or V (odd k)
-  auto dma_one = [&](auto k_tag) __attribute__((always_inline)) {
-    constexpr int K = decltype(k_tag)::value;
-    constexpr int i = K >> 1;
-    if (!dma_on) return;
-    if (KV_FP8 && dma_fp8) {
-      if (K & 1) {
-        st_v[i] = *reinterpret_cast<const uint2*>(dma_vb + ((unsigned long)dma_vo[i] << 4));
-      } else {
-        st_k[i] = *reinterpret_cast<const uint2*>(dma_kb + ((unsigned long)dma_ko[i] << 4));
-        const long so = (long)s_page[KV_FP8 ? dma_sb : 0][KV_FP8 ? 16 * i + lane_row : 0] * p.scale_page_stride +
-                        (long)kvh * p.scale_head_stride;
+  // The whole copy of a tile is issued in one burst at the start of the tile before (handing the
+  // copy instructions out between the MFMAs measured slower).
+  auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
+    const bool ctx = t < Tc;
+    const char* kb = ctx ? kc_lane : kn_lane;
+    const char* vb = ctx ? vc_lane : vn_lane;
+    const unsigned kr = ctx ? cache_row16 : kn_row16;
+    const unsigned vr = ctx ? cache_row16 : vn_row16;
+    char* dst = lds + buf * kBufBytes + wave * 1024;
+    if (KV_FP8 && ctx) {
+#pragma unroll
+      for (int i = 0; i < kDmaGroups; ++i) {
+        st_k[i] = *reinterpret_cast<const uint2*>(kb + ((unsigned long)((unsigned)nslot[i] * kr) << 4));
+        st_v[i] = *reinterpret_cast<const uint2*>(vb + ((unsigned long)((unsigned)nslot[i] * vr) << 4));
+        const long so = (long)(nslot[i] >> p.page_shift) * p.scale_page_stride + (long)kvh * p.scale_head_stride;
         st_ks[i] = p.k_scale[so];
         st_vs[i] = p.v_scale[so];
       }
-    } else if (K & 1) {
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(dma_vb + ((unsigned long)dma_vo[i] << 4)),
-          (__attribute__((address_space(3))) void*)(dma_dst + i * 4096 + kTileBytes), 16, 0, 0);
     } else {
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(dma_kb + ((unsigned long)dma_ko[i] << 4)),
-          (__attribute__((address_space(3))) void*)(dma_dst + i * 4096), 16, 0, 0);
+#pragma unroll
+      for (int i = 0; i < kDmaGroups; ++i) {
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(kb + ((unsigned long)((unsigned)nslot[i] * kr) << 4)),
+            (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(vb + ((unsigned long)((unsigned)nslot[i] * vr) << 4)),
+            (__attribute__((address_space(3))) void*)(dst + i * 4096 + kTileBytes), 16, 0, 0);
+      }
     }
-  };
-  auto dma_all = [&]() __attribute__((always_inline)) {
-#define PDLLM_DMA(K) dma_one(std::integral_constant<int, K>{})
-    PDLLM_DMA(0); PDLLM_DMA(1); PDLLM_DMA(2); PDLLM_DMA(3); PDLLM_DMA(4); PDLLM_DMA(5); PDLLM_DMA(6); PDLLM_DMA(7);
-    PDLLM_DMA(8); PDLLM_DMA(9); PDLLM_DMA(10); PDLLM_DMA(11); PDLLM_DMA(12); PDLLM_DMA(13); PDLLM_DMA(14);
-    PDLLM_DMA(15);
-#undef PDLLM_DMA
   };
   // fp8: dequantise the staged rows into the LDS tile (same layout the direct copies produce)
   auto finish_tile = [&](int t, int buf) __attribute__((always_inline)) {
     if (KV_FP8 && t < Tc) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int ii = i * 4 + wave;
-        char* kdst = lds + buf * kBufBytes + ii * 1024 + lane * 16;
+      for (int i = 0; i < kDmaGroups; ++i) {
+        char* kdst = lds + buf * kBufBytes + (i * 4 + wave) * 1024 + lane * 16;
         *reinterpret_cast<uint4*>(kdst) = dequant_fp8x8(st_k[i].x, st_k[i].y, st_ks[i]);
         *reinterpret_cast<uint4*>(kdst + kTileBytes) = dequant_fp8x8(st_v[i].x, st_v[i].y, st_vs[i]);
       }
@@ -466,19 +474,15 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's direct-to-LDS copies have landed
   };
 
-  const float c = p.scale_log2;
-
   // ---- one pass: row block(s) x NKB key blocks of the tile in LDS ----
-  // DUAL: slot B uses the same key blocks and rides on the operand fragments slot A reads.
+  // dual: slot B uses the same key blocks and rides on the operand fragments slot A reads.
   // Operand reads run two steps ahead of the MFMAs; the scheduling barriers keep that order.
-  // dma_tag: first tile-copy instruction this pass hands out (8 per two-key-block pass), or 16 = none
-  auto pass = [&](bool generic, auto nkb_tag, auto dual_tag, auto dma_tag, bool forA, int kb_first, int bufoff,
+  auto pass = [&](bool generic, auto nkb_tag, auto dual_tag, auto fora_tag, int kb_first, int bufoff,
                   int nvalid, bool active, int a0, int par) __attribute__((always_inline)) {
-    constexpr int DMA0 = decltype(dma_tag)::value;
-    if constexpr (DMA0 < 16) dma_offsets(std::integral_constant<int, DMA0 / 2>{},
-                                         std::integral_constant<int, DMA0 / 2 + 4>{});
     constexpr int NKB = decltype(nkb_tag)::value;
-    constexpr bool DUAL = decltype(dual_tag)::value;
+    constexpr bool DUAL2 = decltype(dual_tag)::value;
+    constexpr bool forA = decltype(fora_tag)::value;
+    constexpr bool QLDS = QB_LDS && !forA;
     const int kbase_bytes = bufoff + kb_first * 32 * kRowBytes;
     const int vbase_bytes = kbase_bytes + kTileBytes;
     bf16x8 (&Q1)[8] = forA ? QA : QB;
@@ -487,41 +491,69 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
     float& l1 = forA ? lA : lB;
     const int srow1 = forA ? srowA : srowB;
 
-    f32x16 S1[NKB], S2[DUAL ? NKB : 1];
+    // the accumulators start at minus the running maximum
+    const float i1 = (M1 == -INFINITY) ? 0.f : -M1;
+    const float i2 = (MB == -INFINITY) ? 0.f : -MB;
+    f32x16 S1[NKB], S2[DUAL2 ? NKB : 1];
 #pragma unroll
     for (int b = 0; b < NKB; ++b)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        S1[b][i] = 0.f;
-        if constexpr (DUAL) S2[b][i] = 0.f;
+        S1[b][i] = i1;
+        if constexpr (DUAL2) S2[b][i] = i2;
       }
-    {
+    if constexpr (!QLDS) {
+      constexpr int PF = 4;  // operand reads run PF steps ahead of the MFMAs (LDS latency ~ 3-4 MFMAs)
+      constexpr int NS = 8 * NKB;
+      unsigned ka[8];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) ka[ks] = lds_base + koff[ks] + kbase_bytes;
+      auto rdk = [&](bf16x8& dst, int stp) __attribute__((always_inline)) {
+        if ((stp >> 3) == 0) lds_read_b128<0>(dst, ka[stp & 7]);
+        else lds_read_b128<32 * kRowBytes>(dst, ka[stp & 7]);
+      };
+      bf16x8 kf[PF];
+#pragma unroll
+      for (int i = 0; i < PF; ++i) rdk(kf[i], i);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int stp = 0; stp < NS; ++stp) {
+        const int kb = stp >> 3, ks = stp & 7;
+        const int young = NS - 1 - stp < PF - 1 ? NS - 1 - stp : PF - 1;  // reads issued after this step's
+        if (young == 3) lds_wait<3>(kf[stp % PF]);
+        else if (young == 2) lds_wait<2>(kf[stp % PF]);
+        else if (young == 1) lds_wait<1>(kf[stp % PF]);
+        else lds_wait<0>(kf[stp % PF]);
+        const bf16x8 cur = kf[stp % PF];
+        S1[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, Q1[ks], S1[kb], 0, 0, 0);
+        if constexpr (DUAL2) S2[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, QB[ks], S2[kb], 0, 0, 0);
+        if (stp + PF < NS) rdk(kf[stp % PF], stp + PF);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+      // shared block next to a slot A: K and Q fragments both come from LDS (compiler-managed reads)
       auto ldk = [&](int stp) __attribute__((always_inline)) {
         const int kb = stp >> 3, ks = stp & 7;
         return *reinterpret_cast<const bf16x8*>(lds + koff[ks] + kbase_bytes + kb * 32 * kRowBytes);
       };
-      bf16x8 kf[2];
-      kf[0] = ldk(0);
-      kf[1] = ldk(1);
+      auto ldq = [&](int stp) __attribute__((always_inline)) {
+        return *reinterpret_cast<const bf16x8*>(dyn_lds + qb_off + (stp & 7) * 1024);
+      };
+      constexpr int PF = 4;
+      bf16x8 kf[PF], qf[PF];
+#pragma unroll
+      for (int i = 0; i < PF; ++i) { kf[i] = ldk(i); qf[i] = ldq(i); }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int stp = 0; stp < 8 * NKB; ++stp) {
-        const int kb = stp >> 3, ks = stp & 7;
-        const bf16x8 cur = kf[stp & 1];
-        S1[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, Q1[ks], S1[kb], 0, 0, 0);
-        if constexpr (DUAL) S2[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, QB[ks], S2[kb], 0, 0, 0);
-        if (stp + 2 < 8 * NKB) kf[stp & 1] = ldk(stp + 2);
-        if constexpr (DMA0 < 16 && NKB == 2) {
-          if (stp == 1) dma_one(std::integral_constant<int, DMA0 + 0>{});
-          if (stp == 5) dma_one(std::integral_constant<int, DMA0 + 1>{});
-          if (stp == 9) dma_one(std::integral_constant<int, DMA0 + 2>{});
-          if (stp == 13) dma_one(std::integral_constant<int, DMA0 + 3>{});
-        }
+        const int kb = stp >> 3;
+        S1[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], qf[stp % PF], S1[kb], 0, 0, 0);
+        if (stp + PF < 8 * NKB) { kf[stp % PF] = ldk(stp + PF); qf[stp % PF] = ldq(stp + PF); }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
 
-    bf16x8 P1[NKB][2], P2[DUAL ? NKB : 1][2];
+    bf16x8 P1[NKB][2], P2[DUAL2 ? NKB : 1][2];
     const bool causal_here = active && p.mask_mode == PDLLM_MASK_CAUSAL;
     const bool dense_here = active && p.mask_mode == PDLLM_MASK_DENSE;
     {
@@ -529,101 +561,90 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
       if (causal_here) { const int cl = srow1 - a0 + 1; lim = cl < lim ? cl : lim; }
       int tl = srow1 - tq_first;
       tl = tl < 0 ? 0 : (tl >= kMaxTok ? kMaxTok - 1 : tl);
-      softmax_update<NKB>(S1, P1, O1, M1, l1, c, h, kb_first, generic, lim,
+      softmax_update<NKB>(S1, P1, O1, M1, l1, h, kb_first, generic, lim,
                           dense_here ? &s_maskbits[par][tl][0] : nullptr);
     }
-    if constexpr (DUAL) {
+    if constexpr (DUAL2) {
       int lim = nvalid;
       if (causal_here) { const int cl = srowB - a0 + 1; lim = cl < lim ? cl : lim; }
       int tl = srowB - tq_first;
       tl = tl < 0 ? 0 : (tl >= kMaxTok ? kMaxTok - 1 : tl);
-      softmax_update<NKB>(S2, P2, OB, MB, lB, c, h, kb_first, generic, lim,
+      softmax_update<NKB>(S2, P2, OB, MB, lB, h, kb_first, generic, lim,
                           dense_here ? &s_maskbits[par][tl][0] : nullptr);
     }
     __builtin_amdgcn_sched_barrier(0);
     {
       typedef __attribute__((ext_vector_type(8))) short s16x8;
-      // step = (kb, j, db): V^T fragment of keys 32 kb + 16 j .. +16, columns 32 db .. +32
-      auto ldv = [&](int stp, int r) __attribute__((always_inline)) {
+      constexpr int NS = 8 * NKB;
+      // step = (kj, db): V^T fragment of keys 16 kj .. +16 of the pass, columns 32 db .. +32
+      unsigned va[2][4];
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int db = 0; db < 4; ++db) va[r][db] = lds_base + voff[r][db] + vbase_bytes;
+      auto rdv = [&](s16x4& dst, int stp, int r) __attribute__((always_inline)) {
         const int db = stp & 3, kj = stp >> 2;
-        return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_s16x4*)(lds + voff[r][db] + vbase_bytes + kj * 16 * kRowBytes));
+        if (kj == 0) lds_read_tr16_b64<0>(dst, va[r][db]);
+        else if (kj == 1) lds_read_tr16_b64<16 * kRowBytes>(dst, va[r][db]);
+        else if (kj == 2) lds_read_tr16_b64<32 * kRowBytes>(dst, va[r][db]);
+        else lds_read_tr16_b64<48 * kRowBytes>(dst, va[r][db]);
       };
       s16x4 lo[2], hi[2];
-      lo[0] = ldv(0, 0); hi[0] = ldv(0, 1);
-      lo[1] = ldv(1, 0); hi[1] = ldv(1, 1);
+      rdv(lo[0], 0, 0); rdv(hi[0], 0, 1);
+      rdv(lo[1], 1, 0); rdv(hi[1], 1, 1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int stp = 0; stp < 8 * NKB; ++stp) {
+      for (int stp = 0; stp < NS; ++stp) {
         const int db = stp & 3, kj = stp >> 2;
+        if (stp + 1 < NS) lds_wait2<2>(lo[stp & 1], hi[stp & 1]);
+        else lds_wait2<0>(lo[stp & 1], hi[stp & 1]);
         const s16x4 a = lo[stp & 1], b2 = hi[stp & 1];
         const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
         const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
         O1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P1[kj >> 1][kj & 1], O1[db], 0, 0, 0);
-        if constexpr (DUAL) OB[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P2[kj >> 1][kj & 1], OB[db], 0, 0, 0);
-        if (stp + 2 < 8 * NKB) { lo[stp & 1] = ldv(stp + 2, 0); hi[stp & 1] = ldv(stp + 2, 1); }
-        if constexpr (DMA0 < 16 && NKB == 2) {
-          if (stp == 1) dma_one(std::integral_constant<int, DMA0 + 4>{});
-          if (stp == 5) dma_one(std::integral_constant<int, DMA0 + 5>{});
-          if (stp == 9) dma_one(std::integral_constant<int, DMA0 + 6>{});
-          if (stp == 13) dma_one(std::integral_constant<int, DMA0 + 7>{});
-        }
+        if constexpr (DUAL2) OB[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P2[kj >> 1][kj & 1], OB[db], 0, 0, 0);
+        if (stp + 2 < NS) { rdv(lo[stp & 1], stp + 2, 0); rdv(hi[stp & 1], stp + 2, 1); }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
 
-  using I0 = std::integral_constant<int, 0>;
-  using I8 = std::integral_constant<int, 8>;
-  using I16 = std::integral_constant<int, 16>;
-  auto compute = [&](bool gen_tag, int t, int buf, bool has_next, int sb_next) __attribute__((always_inline)) {
+  auto compute = [&](bool generic, int t, int buf, bool has_next) __attribute__((always_inline)) {
     const int bufoff = buf * kBufBytes;
     const bool active = t >= Tc;
     const int a0 = active ? (t - Tc) * kKT : 0;
     int nvalid = active ? Sa - a0 : ctx_total - t * kKT;
     nvalid = nvalid < kKT ? nvalid : kKT;
     using N1 = std::integral_constant<int, 1>;
-    using N2 = std::integral_constant<int, 2>;
-    using Dual = std::integral_constant<bool, NB == 4>;
+    using NT = std::integral_constant<int, kNKB>;
+    using Dual = std::integral_constant<bool, DUAL>;
     using Single = std::integral_constant<bool, false>;
-    if (has_next) {
-      // the whole copy of the next tile is issued up front (the copy instructions are scheduling
-      // boundaries; spreading them through the MFMA loops measured slower)
-      dma_begin(t + 1, sb_next, buf ^ 1, true);
-      dma_offsets(I0{}, I8{});
-      dma_all();
+    if (has_next) issue_tile(t + 1, buf ^ 1);
+    if (t + 2 < T1) load_slots(t + 2);
+    if (HAS_A) pass(generic, NT{}, Dual{}, std::true_type{}, 0, bufoff, nvalid, active, a0, buf);
+    if (HAS_B && !DUAL) {
+      if (GS == 2 || ((t & 1) == parB))
+        pass(generic, N1{}, Single{}, std::false_type{}, kbB, bufoff, nvalid, active, a0, buf);
     }
-    if (HAS_A) {
-      pass(gen_tag, N2{}, Dual{}, I16{}, true, 0, bufoff, nvalid, active, a0, buf);
-      pass(gen_tag, N2{}, Dual{}, I16{}, true, 2, bufoff, nvalid, active, a0, buf);
-    }
-    if (NB == 1) pass(gen_tag, N1{}, Single{}, I16{}, false, kb0, bufoff, nvalid, active, a0, buf);
-    if (NB == 2) pass(gen_tag, N2{}, Single{}, I16{}, false, kb0, bufoff, nvalid, active, a0, buf);
   };
 
   auto step = [&](int t) __attribute__((always_inline)) {
     const int rel = t - T0;
     const int buf = rel & 1;
-    if (t + 2 < T1) resolve_begin(t + 2);
     if (t + 1 < T1) build_mask(t + 1, buf ^ 1);
     const bool active = t >= Tc;
     const int a0 = active ? (t - Tc) * kKT : 0;
     const int nv = active ? Sa - a0 : ctx_total - t * kKT;
     const bool generic = nv < kKT || (active && p.mask_mode != PDLLM_MASK_FULL);
-    compute(generic, t, buf, t + 1 < T1, (rel + 1) % 3);
-    if (t + 2 < T1) resolve_end(t + 2, (rel + 2) % 3);
+    compute(generic, t, buf, t + 1 < T1);
     if (t + 1 < T1) finish_tile(t + 1, buf ^ 1);
     __syncthreads();
   };
 
   if (T0 < T1) {
-    resolve_begin(T0);
-    resolve_end(T0, 0);
-    if (T0 + 1 < T1) { resolve_begin(T0 + 1); resolve_end(T0 + 1, 1); }
-    __syncthreads();
-    dma_begin(T0, 0, 0, true);
-    dma_offsets(I0{}, I8{});
-    dma_all();
+    load_slots(T0);
+    issue_tile(T0, 0);  // waits for the slots it uses
+    if (T0 + 1 < T1) load_slots(T0 + 1);
     build_mask(T0, 0);
     finish_tile(T0, 0);
     __syncthreads();
@@ -636,8 +657,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
     const int tq = ridx / G;
     const int g = ridx - tq * G;
     const float inv = lfin > 0.f ? 1.f / lfin : 0.f;
-    if (p.num_splits == 1) {
-      __bf16* op = p.out + (long)(q0 + tq) * p.o_stride + (long)(kvh * G + g) * kD + 32 * db + 4 * h;
+    if (whole) {
+      __bf16* op = p.out + (long)(q0 + tq) * p.o_stride + (long)(kvh * G + g) * kD + 32 * db + 4 * he;
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         uint2 w;
@@ -646,14 +667,14 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
         *reinterpret_cast<uint2*>(op + 8 * i4) = w;
       }
     } else {
-      const long R = ((long)(q0 + tq) * p.Hq + kvh * G + g) * p.num_splits + split;
-      float* wp = p.ws_o + R * kD + 32 * db + 4 * h;
+      const long R = ((long)(q0 + tq) * p.Hq + kvh * G + g) * p.max_pieces + piece;
+      float* wp = p.ws_o + R * kD + 32 * db + 4 * he;
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         float4 w = {o[4 * i4 + 0] * inv, o[4 * i4 + 1] * inv, o[4 * i4 + 2] * inv, o[4 * i4 + 3] * inv};
         *reinterpret_cast<float4*>(wp + 8 * i4) = w;
       }
-      if (db == 0 && h == 0) p.ws_lse[R] = lfin > 0.f ? mfin + __log2f(lfin) : -INFINITY;  // log2 domain
+      if (db == 0 && he == 0) p.ws_lse[R] = lfin > 0.f ? mfin + __log2f(lfin) : -INFINITY;  // log2 domain
     }
   };
 
@@ -662,37 +683,38 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
 #pragma unroll
     for (int db = 0; db < 4; ++db) emit(ridxA, db, OA[db], MA, lA);
   }
-  if (NB > 0) {
+  if (HAS_B) {
     lB = half_swap_sum(lB);
     if (GS == 1) {
 #pragma unroll
       for (int db = 0; db < 4; ++db) emit(ridxB, db, OB[db], MB, lB);
     } else {
-      // merge the GS partial results of a shared block through LDS (the tile buffers are free now)
+      // merge the GS partial results of a shared block through LDS (the tile buffers are free now);
+      // element (d, row) of a partial lives at [d][row ^ (d & 31)], conflict-free both ways
       float* part = reinterpret_cast<float*>(lds) + wave * (kPartBytes / 4);
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int d = 32 * db + 8 * (i >> 2) + 4 * h + (i & 3);
-          part[d * kPartStride + l32] = OB[db][i];
+          const int d = 32 * db + 8 * (i >> 2) + 4 * he + (i & 3);
+          part[d * 32 + (l32e ^ (d & 31))] = OB[db][i];
         }
-      if (h == 0) {
-        s_ml[wave][0][l32] = MB;
-        s_ml[wave][1][l32] = lB;
+      if (he == 0) {
+        s_ml[wave][0][l32e] = MB;
+        s_ml[wave][1][l32e] = lB;
       }
       __syncthreads();
       const int wbase = wave - gi;
       float M = -INFINITY;
 #pragma unroll
-      for (int w = 0; w < GS; ++w) M = fmaxf(M, s_ml[wbase + w][0][l32]);
+      for (int w = 0; w < GS; ++w) M = fmaxf(M, s_ml[wbase + w][0][l32e]);
       const float Muse = (M == -INFINITY) ? 0.f : M;
       float wgt[GS];
       float L = 0.f;
 #pragma unroll
       for (int w = 0; w < GS; ++w) {
-        wgt[w] = __builtin_amdgcn_exp2f(s_ml[wbase + w][0][l32] - Muse);
-        L += wgt[w] * s_ml[wbase + w][1][l32];
+        wgt[w] = __builtin_amdgcn_exp2f(s_ml[wbase + w][0][l32e] - Muse);
+        L += wgt[w] * s_ml[wbase + w][1][l32e];
       }
       constexpr int NDB = 4 / GS;  // column blocks this wave finishes
 #pragma unroll
@@ -706,51 +728,120 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnKParams p)
           const float* pw = reinterpret_cast<const float*>(lds) + (wbase + w) * (kPartBytes / 4);
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            const int d = 32 * db + 8 * (i >> 2) + 4 * h + (i & 3);
-            acc[i] += wgt[w] * pw[d * kPartStride + l32];
+            const int d = 32 * db + 8 * (i >> 2) + 4 * he + (i & 3);
+            acc[i] += wgt[w] * pw[d * 32 + (l32e ^ (d & 31))];
           }
         }
         emit(ridxB, db, acc, M, L);
       }
     }
   }
+  __syncthreads();  // the next piece reuses the LDS buffers
+  }  // pieces
 }
 
-// Reduce the split-KV partials: one wave per (token, q-head) row.
-__global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ ws_o,
-                                                         const float* __restrict__ ws_lse,
-                                                         __bf16* __restrict__ out, long o_stride,
-                                                         const int* __restrict__ q_start_loc,
-                                                         int n_req, int max_q_len, int Hq,
-                                                         int num_splits, long n_tokens) {
-  const int lane = threadIdx.x & 63;
-  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const long per_req = (long)max_q_len * Hq;
-  if (row >= per_req * n_req) return;
+// Slot table: for request r and v < count(r), table[r][v] = page * page_size + offset of the v-th
+// visible prefix key (ranges in order, each mapped through the page table); entries up to the
+// next multiple of the tile size repeat the first key of their tile (they are loaded but
+// masked); table[r][stride - 1] = count(r) = min(sum of range lengths, max_ctx_len).
+// Page ids outside [0, n_pages) are clamped, so a slot never points outside the cache.
+__global__ __launch_bounds__(256) void attn_slot_table_kernel(const AttnKParams p, int* __restrict__ table) {
+  __shared__ int s_cum[kMaxRanges + 1];
+  __shared__ int s_start[kMaxRanges];
+  __shared__ int s_len[kMaxRanges];
+  const int tid = threadIdx.x;
+  const int req = blockIdx.y;
+  const int r0 = p.range_ptr[req];
+  int nr = p.range_ptr[req + 1] - r0;
+  nr = nr < 0 ? 0 : (nr > kMaxRanges ? kMaxRanges : nr);
+  if (tid < nr) {
+    const int len = p.range_len[r0 + tid];
+    s_len[tid] = len > 0 ? len : 0;
+    s_start[tid] = p.range_start[r0 + tid];
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int cc = 0;
+    for (int i = 0; i < nr; ++i) { s_cum[i] = cc; cc += s_len[i]; }
+    s_cum[nr] = cc;
+  }
+  __syncthreads();
+  const int count = s_cum[nr] < p.max_ctx_len ? s_cum[nr] : p.max_ctx_len;
+  int* row = table + (long)req * p.slot_stride;
+  if (blockIdx.x == 0 && tid == 0) row[p.slot_stride - 1] = count;
+  const int padded = (count + kKT - 1) / kKT * kKT;
+  const int v = blockIdx.x * 256 + tid;
+  if (v >= padded) return;
+  const int vv = v < count ? v : (v / kKT) * kKT;
+  int rp = 0;
+  while (rp + 1 < nr && vv >= s_cum[rp + 1]) ++rp;
+  const int tok = s_start[rp] + (vv - s_cum[rp]);
+  int pi = tok >> p.page_shift;
+  pi = pi < 0 ? 0 : (pi >= p.bt_stride ? p.bt_stride - 1 : pi);
+  int page = p.block_table[(long)req * p.bt_stride + pi];
+  page = page < 0 ? 0 : (page >= p.n_pages ? p.n_pages - 1 : page);
+  row[v] = (page << p.page_shift) + (tok & ((1 << p.page_shift) - 1));
+}
+
+// Reduce the partial results of the columns that were cut into several pieces: one wave per
+// (token, q-head) row.  Rows of a column with a single piece were written directly.
+struct MergeParams {
+  const float* ws_o;
+  const float* ws_lse;
+  __bf16* out;
+  const int* q_start_loc;
+  long o_stride, n_tokens;
+  int n_req, max_q_len, Hq, Hkv, rows_per_group, row_tiles, t_lin, span, max_pieces;
+};
+
+__global__ __launch_bounds__(256) void attn_merge_kernel(const MergeParams m) {
+  // 32 lanes per row (4 columns each), 8 rows per workgroup
+  const int l = threadIdx.x & 31;
+  const long row = (long)blockIdx.x * 8 + (threadIdx.x >> 5);
+  const long per_req = (long)m.max_q_len * m.Hq;
+  if (row >= per_req * m.n_req) return;
   const int req = (int)(row / per_req);
   const int rem = (int)(row - (long)req * per_req);
-  const int tq = rem / Hq;
-  const int head = rem - tq * Hq;
-  const int q0 = q_start_loc[req];
-  const int Sq = q_start_loc[req + 1] - q0;
-  if (q0 < 0 || tq >= Sq || (long)q0 + Sq > n_tokens || Sq > max_q_len) return;
-  const long R = ((long)(q0 + tq) * Hq + head) * num_splits;
+  const int tq = rem / m.Hq;
+  const int head = rem - tq * m.Hq;
+  const int q0 = m.q_start_loc[req];
+  const int Sq = m.q_start_loc[req + 1] - q0;
+  if (q0 < 0 || tq >= Sq || (long)q0 + Sq > m.n_tokens || Sq > m.max_q_len) return;
+  const int G = m.Hq / m.Hkv;
+  const int kvh = head / G;
+  const int col = (req * m.Hkv + kvh) * m.row_tiles + (tq * G + (head - kvh * G)) / m.rows_per_group;
+  const int first = (col * m.t_lin) / m.span;
+  const int np = ((col + 1) * m.t_lin - 1) / m.span - first + 1;
+  if (np == 1) return;
+  const long R = ((long)(q0 + tq) * m.Hq + head) * m.max_pieces;
   float M = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, ws_lse[R + s]);
-  float2 acc = {0.f, 0.f};
+  for (int s = 0; s < np; ++s) M = fmaxf(M, m.ws_lse[R + s]);
+  float4 acc = {0.f, 0.f, 0.f, 0.f};
   float L = 0.f;
   if (M > -INFINITY) {
-    for (int s = 0; s < num_splits; ++s) {
-      const float w = __builtin_amdgcn_exp2f(ws_lse[R + s] - M);
-      const float2 o = *reinterpret_cast<const float2*>(ws_o + (R + s) * kD + 2 * lane);
-      acc.x += w * o.x;
-      acc.y += w * o.y;
-      L += w;
+    for (int s0 = 0; s0 < np; s0 += 4) {
+      float w[4];
+      float4 o[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const bool on = s0 + u < np;
+        const float lse = on ? m.ws_lse[R + s0 + u] : -INFINITY;
+        w[u] = lse == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(lse - M);  // empty piece: weight 0, not read
+        o[u] = w[u] > 0.f ? *reinterpret_cast<const float4*>(m.ws_o + (R + s0 + u) * kD + 4 * l)
+                          : float4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        acc.x += w[u] * o[u].x; acc.y += w[u] * o[u].y; acc.z += w[u] * o[u].z; acc.w += w[u] * o[u].w;
+        L += w[u];
+      }
     }
   }
   const float inv = L > 0.f ? 1.f / L : 0.f;
-  *reinterpret_cast<uint32_t*>(out + (long)(q0 + tq) * o_stride + (long)head * kD + 2 * lane) =
-      pack_bf16x2(acc.x * inv, acc.y * inv);
+  uint2 packed;
+  packed.x = pack_bf16x2(acc.x * inv, acc.y * inv);
+  packed.y = pack_bf16x2(acc.z * inv, acc.w * inv);
+  *reinterpret_cast<uint2*>(m.out + (long)(q0 + tq) * m.o_stride + (long)head * kD + 4 * l) = packed;
 }
 
 // ---------------------------------------------------------------------------
@@ -759,8 +850,12 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict
 
 struct AttnPlan {
   int J;
-  int num_splits;
   int row_tiles;
+  int t_lin;       // positions per column on the tile line
+  int span;        // tiles per workgroup
+  int n_lin;       // columns * t_lin
+  int max_pieces;  // most pieces a column is cut into
+  int grid;        // workgroups
 };
 
 static int ilog2_exact(int v) {
@@ -768,6 +863,11 @@ static int ilog2_exact(int v) {
   int s = 0;
   while ((1 << s) < v) ++s;
   return s;
+}
+
+// ints per request of the slot table: the keys padded to whole tiles, one spare tile, the count
+static int64_t slot_table_stride_for(const pdllm_attn_desc* d) {
+  return ((int64_t)d->max_ctx_len + kKT - 1) / kKT * kKT + kKT;
 }
 
 static int validate_desc(const pdllm_attn_desc* d, bool prefill) {
@@ -807,7 +907,10 @@ static int validate_desc(const pdllm_attn_desc* d, bool prefill) {
     const uintptr_t palign = d->kv_dtype == PDLLM_KV_FP8_E4M3 ? 8 : 16;
     if (((uintptr_t)d->k_cache | (uintptr_t)d->v_cache) % palign) return PDLLM_ERR_STRIDE;
   }
-  if (d->num_splits < 0 || d->num_splits > 64) return PDLLM_ERR_SHAPE;
+  if (has_cache && d->slot_table != nullptr) {
+    if (d->slot_table_stride < slot_table_stride_for(d) || ((uintptr_t)d->slot_table % 4)) return PDLLM_ERR_STRIDE;
+  }
+  if (d->num_splits < 0 || d->num_splits > 16 || d->tiles_per_workgroup < 0) return PDLLM_ERR_SHAPE;
   if (d->rows_per_group != 0) {
     const int j = d->rows_per_group / 32;
     if (d->rows_per_group % 32 || !(j == 1 || j == 2 || j == 4 || j == 5 || j == 6 || j == 8)) return PDLLM_ERR_SHAPE;
@@ -815,9 +918,23 @@ static int validate_desc(const pdllm_attn_desc* d, bool prefill) {
   return PDLLM_OK;
 }
 
-// Pick the row-group size J and the number of KV splits: minimise the modelled
-// makespan (rounds of workgroups over 256 CUs x key tiles x row blocks per wave,
-// floored by the cost of staging a tile) plus the HBM cost of split partials.
+// Bytes of dynamic LDS of attn_fwd_kernel<*, J>: Q fragments of the shared blocks next to a
+// slot A, then the bit rows of a dense mask.
+static int dyn_lds_bytes(int J, int mask_mode) {
+  int b = (J == 5 || J == 6) ? (J - 4) * 8192 : 0;
+  if (mask_mode == PDLLM_MASK_DENSE) b += 2 * kMaxTok * kNKB * 4;
+  return b;
+}
+
+// Pick the row-group size J and the span (tiles per workgroup) by a small cost model.
+// All tiles of all columns (request, KV head, row group) lie on one line of n_cols * t_lin
+// positions; workgroup g takes positions [g * span, (g + 1) * span).  span = t_lin gives one
+// workgroup per column; a smaller span that does not divide t_lin lets pieces of two columns
+// share a workgroup, which balances any shape over the CUs at the price of fp32 partials.
+// Unit of time: one wave doing one 32-row block of one 64-key tile on a CU of its own.  A
+// workgroup alone on a CU spends (fixed + blocks per wave) per tile; two workgroups sharing a CU
+// (bf16 cache, LDS footprint <= 80 KB) overlap matrix and vector work and take kPair of the
+// serial time.  The most loaded CU sets the makespan.
 static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   const int G = d->num_q_heads / d->num_kv_heads;
   const long rows = (long)d->max_q_len * G;
@@ -825,57 +942,129 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   const long ctx = prefill ? 0 : d->max_ctx_len;
   const long T = (ctx + kKT - 1) / kKT + (d->max_q_len + kKT - 1) / kKT;
   const long units = (long)d->n_req * d->num_kv_heads;
+  const bool fp8 = !prefill && d->k_cache != nullptr && d->max_ctx_len > 0 && d->kv_dtype == PDLLM_KV_FP8_E4M3;
   const int cus = 256;
+  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 1.5;
+  constexpr int kStaticLds = 66 * 1024;
   static const int js[] = {1, 2, 4, 5, 6, 8};
-  AttnPlan best = {4, 1, 1};
+  static const double upw[] = {0.25, 0.5, 1.0, 1.25, 1.5, 2.0};
+  AttnPlan best = {4, 1, (int)T, (int)T, (int)T, 1, 1};
   double best_cost = 1e300;
   for (int ji = 0; ji < 6; ++ji) {
     const int J = js[ji];
     if (d->rows_per_group && d->rows_per_group != 32 * J) continue;
-    if (!d->rows_per_group && J == 8) continue;  // two full row blocks per wave spill registers: only on request
+    if (!d->rows_per_group && (J == 5 || J == 6 || J == 8)) continue;  // too many registers for two workgroups per CU: only on request
     const long row_tiles = (nblk + J - 1) / J;
-    const int max_splits = prefill ? 1 : 16;
-    for (int S = 1; S <= max_splits; ++S) {
-      if (d->num_splits && d->num_splits != S) continue;
-      if (S > 1 && S > T) break;
-      const long wgs = units * row_tiles * S;
-      const int per_cu = 1;  // 128 KB of LDS tile buffers: one workgroup per CU
-      const double rounds = (double)((wgs + (long)cus * per_cu - 1) / ((long)cus * per_cu));
-      const double tiles = (double)((T + S - 1) / S);
-      double per_tile = J / 4.0;           // MFMA block-tiles per wave per key tile
-      if (per_tile < 0.6) per_tile = 0.6;  // staging / barrier floor
-      double cost = rounds * per_cu * tiles * per_tile;
-      if (S > 1) {
-        // fp32 partial write + read, in units of "key tile of one wave" (~1024 cycles)
-        const double part_bytes = (double)units * rows * S * (kD + 1) * 4.0 * 2.0;
-        cost += part_bytes / (8e12 / 2.4e9 * 1024.0) + 4.0;
+    const long cols = units * row_tiles;
+    const bool two = !fp8 && J != 8 && kStaticLds + dyn_lds_bytes(J, d->mask_mode) <= 80 * 1024;
+    const long slots = (long)cus * (two ? 2 : 1);
+    // candidate spans: whole columns, columns cut into 2..16 equal parts, and the balanced cut
+    for (int cand = 0; cand <= 18; ++cand) {
+      long t_lin = T, span;
+      if (cand == 0) {
+        span = T;
+      } else if (cand <= 15) {
+        const int S = cand + 1;
+        if (S > T) break;
+        span = (T + S - 1) / S;
+        t_lin = span * S;  // aligned: pieces never cross a column
+      } else if (cand == 16) {
+        if (prefill) continue;
+        span = (cols * T + slots - 1) / slots;
+        if (span >= T || span < 2) continue;
+      } else if (cand == 17) {
+        if (prefill) continue;
+        span = (cols * T + 2 * slots - 1) / (2 * slots);
+        if (span >= T || span < 4) continue;
+      } else {
+        if (d->tiles_per_workgroup <= 0) continue;
+        span = d->tiles_per_workgroup < T ? d->tiles_per_workgroup : T;
+      }
+      if (d->tiles_per_workgroup > 0) {
+        if (cand != 18) continue;
+      } else if (d->num_splits) {
+        if (cand == 0 ? d->num_splits != 1 : (cand > 15 || d->num_splits != cand + 1)) continue;
+      } else if (prefill && cand != 0) {
+        continue;
+      }
+      const long n_lin = cols * t_lin;
+      if (n_lin >= (1l << 30)) continue;
+      const long grid = (n_lin + span - 1) / span;
+      const long n = (grid + cus - 1) / cus;  // workgroups on the most loaded CU
+      const double serial = two ? (double)(n / 2) * 2.0 * kPair + (double)(n % 2) : (double)n;
+      const bool cut = span < t_lin;
+      const long pieces = cut ? (t_lin + span - 1) / span + (t_lin % span ? 1 : 0) : 1;
+      double cost = serial * ((double)span * (kFixed + upw[ji]) + kPiece * (cut && t_lin % span ? 2.0 : 1.0)) + 1.0;
+      if (cut) {
+        // fp32 partials written and read back (~4 MB per unit of time), plus the merge launch
+        const double avg_pieces = (double)t_lin / (double)span + (t_lin % span ? 1.0 : 0.0);
+        const double part_bytes = (double)units * rows * avg_pieces * (kD + 1) * 4.0 * 2.0;
+        cost += part_bytes / 4.0e6 + 4.0;
       }
       if (cost < best_cost) {
         best_cost = cost;
         best.J = J;
-        best.num_splits = S;
         best.row_tiles = (int)row_tiles;
+        best.t_lin = (int)t_lin;
+        best.span = (int)span;
+        best.n_lin = (int)n_lin;
+        best.max_pieces = (int)pieces;
+        best.grid = (int)grid;
       }
     }
+  }
+  if (best_cost == 1e300) {
+    // the forced values fit no candidate (e.g. a split of a prefill): one workgroup per column, J = 4
+    const long row_tiles = (nblk + 3) / 4;
+    best = {4, (int)row_tiles, (int)T, (int)T, (int)(units * row_tiles * T), 1, (int)(units * row_tiles)};
   }
   return best;
 }
 
-static int64_t ws_bytes_for(const pdllm_attn_desc* d, int num_splits) {
-  if (num_splits <= 1) return 0;
+static bool needs_own_table(const pdllm_attn_desc* d, bool prefill) {
+  return !prefill && d->k_cache != nullptr && d->max_ctx_len > 0 && d->slot_table == nullptr;
+}
+
+// split-KV partials first, then (when the caller passed no slot table) the table
+static int64_t partial_bytes_for(const pdllm_attn_desc* d, int max_pieces) {
+  if (max_pieces <= 1) return 0;
   const int64_t rows = d->n_tokens * d->num_q_heads;
-  return rows * num_splits * (int64_t)(kD + 1) * 4;
+  return rows * max_pieces * (int64_t)(kD + 1) * 4;
+}
+static int64_t ws_bytes_for(const pdllm_attn_desc* d, int max_pieces, bool prefill) {
+  int64_t b = partial_bytes_for(d, max_pieces);
+  if (needs_own_table(d, prefill)) b += (int64_t)d->n_req * slot_table_stride_for(d) * 4;
+  return b;
+}
+
+static void fill_table_params(const pdllm_attn_desc* d, AttnKParams& p) {
+  p.block_table = d->block_table;
+  p.range_ptr = d->range_ptr;
+  p.range_start = d->range_start;
+  p.range_len = d->range_len;
+  p.bt_stride = d->bt_stride;
+  p.n_pages = (int)d->n_pages;
+  p.page_shift = ilog2_exact(d->page_size);
+  p.max_ctx_len = d->max_ctx_len;
+  p.max_ranges = d->max_ranges;
+}
+
+static int launch_slot_table(const AttnKParams& p, int n_req, int* table, hipStream_t stream) {
+  const int padded = (p.max_ctx_len + kKT - 1) / kKT * kKT;
+  const dim3 grid((unsigned)((padded + 255) / 256), (unsigned)n_req);
+  hipLaunchKernelGGL(attn_slot_table_kernel, grid, dim3(256), 0, stream, p, table);
+  return launch_status();
 }
 
 static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t stream) {
   int st = validate_desc(d, prefill);
   if (st != PDLLM_OK) return st;
   const AttnPlan plan = make_plan(d, prefill);
-  const int64_t need = ws_bytes_for(d, plan.num_splits);
+  const int64_t need = ws_bytes_for(d, plan.max_pieces, prefill);
   if (need > 0 && (!d->workspace || d->workspace_bytes < need)) return PDLLM_ERR_WORKSPACE;
   if (need > 0 && ((uintptr_t)d->workspace % 16)) return PDLLM_ERR_STRIDE;
 
-  AttnKParams p;
+  AttnKParams p = {};
   p.q = static_cast<const __bf16*>(d->q);
   p.k_new = static_cast<const __bf16*>(d->k_new);
   p.v_new = static_cast<const __bf16*>(d->v_new);
@@ -885,42 +1074,50 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
   p.v_cache = has_cache ? d->v_cache : nullptr;
   p.k_scale = d->k_scale;
   p.v_scale = d->v_scale;
-  p.block_table = d->block_table;
   p.q_start_loc = d->q_start_loc;
-  p.range_ptr = has_cache ? d->range_ptr : nullptr;
-  p.range_start = d->range_start;
-  p.range_len = d->range_len;
   p.mask = d->mask_mode == PDLLM_MASK_DENSE ? d->mask : nullptr;
   const int64_t rows = d->n_tokens * d->num_q_heads;
-  p.ws_o = static_cast<float*>(d->workspace);
-  p.ws_lse = p.ws_o ? p.ws_o + rows * plan.num_splits * kD : nullptr;
+  p.ws_o = plan.max_pieces > 1 ? static_cast<float*>(d->workspace) : nullptr;
+  p.ws_lse = p.ws_o ? p.ws_o + rows * plan.max_pieces * kD : nullptr;
+  if (has_cache) {
+    fill_table_params(d, p);
+    p.slot_stride = d->slot_table ? d->slot_table_stride : slot_table_stride_for(d);
+    if (d->slot_table) {
+      p.slot_table = d->slot_table;
+    } else {
+      int* table = reinterpret_cast<int*>(static_cast<char*>(d->workspace) + partial_bytes_for(d, plan.max_pieces));
+      st = launch_slot_table(p, d->n_req, table, stream);
+      if (st != PDLLM_OK) return st;
+      p.slot_table = table;
+    }
+  }
   p.q_stride = d->q_stride; p.kn_stride = d->kn_stride; p.vn_stride = d->vn_stride; p.o_stride = d->o_stride;
   p.cache_page_stride = d->cache_page_stride;
   p.cache_token_stride = d->cache_token_stride;
   p.cache_head_stride = d->cache_head_stride;
   p.mask_stride = d->mask_stride;
   p.n_tokens = d->n_tokens;
-  p.n_pages = (int)d->n_pages;
-  p.bt_stride = d->bt_stride;
   p.scale_page_stride = d->scale_page_stride;
   p.scale_head_stride = d->scale_head_stride;
   p.n_req = d->n_req; p.Hq = d->num_q_heads; p.Hkv = d->num_kv_heads; p.G = d->num_q_heads / d->num_kv_heads;
-  p.page_shift = has_cache ? ilog2_exact(d->page_size) : 0;
   p.mask_mode = d->mask_mode;
   p.J = plan.J;
   p.row_tiles = plan.row_tiles;
-  p.num_splits = plan.num_splits;
+  p.t_lin = plan.t_lin;
+  p.span = plan.span;
+  p.n_lin = plan.n_lin;
+  p.max_pieces = plan.max_pieces;
   p.max_q_len = d->max_q_len;
   p.scale_log2 = d->sm_scale * 1.4426950408889634f;
 
-  const long nblocks = (long)d->n_req * d->num_kv_heads * plan.row_tiles * plan.num_splits;
-  if (nblocks <= 0 || nblocks > 0x7fffffffL) return PDLLM_ERR_SHAPE;
-  const dim3 grid((unsigned)nblocks), block(kThreads);
+  if (plan.grid <= 0) return PDLLM_ERR_SHAPE;
+  const dim3 grid((unsigned)plan.grid), block(kThreads);
   const bool fp8 = has_cache && d->kv_dtype == PDLLM_KV_FP8_E4M3;
+  const int dyn = dyn_lds_bytes(plan.J, d->mask_mode);
 #define PDLLM_LAUNCH(JJ)                                                                              \
   do {                                                                                                \
-    if (fp8) hipLaunchKernelGGL((attn_fwd_kernel<1, JJ>), grid, block, 0, stream, p);                 \
-    else hipLaunchKernelGGL((attn_fwd_kernel<0, JJ>), grid, block, 0, stream, p);                     \
+    if (fp8) hipLaunchKernelGGL((attn_fwd_kernel<1, JJ>), grid, block, dyn, stream, p);               \
+    else hipLaunchKernelGGL((attn_fwd_kernel<0, JJ>), grid, block, dyn, stream, p);                   \
   } while (0)
   switch (plan.J) {
     case 1: PDLLM_LAUNCH(1); break;
@@ -934,11 +1131,15 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
 #undef PDLLM_LAUNCH
   st = launch_status();
   if (st != PDLLM_OK) return st;
-  if (plan.num_splits > 1) {
+  if (plan.max_pieces > 1) {
+    MergeParams m;
+    m.ws_o = p.ws_o; m.ws_lse = p.ws_lse; m.out = p.out; m.q_start_loc = p.q_start_loc;
+    m.o_stride = p.o_stride; m.n_tokens = p.n_tokens;
+    m.n_req = p.n_req; m.max_q_len = p.max_q_len; m.Hq = p.Hq; m.Hkv = p.Hkv;
+    m.rows_per_group = 32 * plan.J; m.row_tiles = plan.row_tiles;
+    m.t_lin = plan.t_lin; m.span = plan.span; m.max_pieces = plan.max_pieces;
     const long mrows = (long)d->n_req * d->max_q_len * d->num_q_heads;
-    hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((mrows + 3) / 4)), dim3(256), 0, stream,
-                       p.ws_o, p.ws_lse, p.out, p.o_stride, p.q_start_loc, p.n_req, p.max_q_len,
-                       p.Hq, p.num_splits, p.n_tokens);
+    hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((mrows + 7) / 8)), dim3(256), 0, stream, m);
     st = launch_status();
   }
   return st;
@@ -949,7 +1150,28 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
 extern "C" int64_t pdllm_attn_workspace_bytes(const pdllm_attn_desc* desc) {
   const int st = pdllm::validate_desc(desc, false);
   if (st != PDLLM_OK) return st;
-  return pdllm::ws_bytes_for(desc, pdllm::make_plan(desc, false).num_splits);
+  return pdllm::ws_bytes_for(desc, pdllm::make_plan(desc, false).max_pieces, false);
+}
+
+extern "C" int64_t pdllm_attn_slot_table_stride(const pdllm_attn_desc* desc) {
+  if (!desc) return PDLLM_ERR_NULL;
+  if (desc->max_ctx_len < 0) return PDLLM_ERR_SHAPE;
+  return pdllm::slot_table_stride_for(desc);
+}
+
+extern "C" int pdllm_attn_build_slot_table(const pdllm_attn_desc* desc, int32_t* table, int64_t table_stride,
+                                           pdllm_stream_t stream) {
+  if (!desc || !table) return PDLLM_ERR_NULL;
+  if (!desc->block_table || !desc->range_ptr || !desc->range_start || !desc->range_len) return PDLLM_ERR_NULL;
+  if (desc->n_req <= 0 || desc->max_ctx_len <= 0 || desc->bt_stride <= 0) return PDLLM_ERR_SHAPE;
+  if (pdllm::ilog2_exact(desc->page_size) < 0) return PDLLM_ERR_SHAPE;
+  if (desc->n_pages <= 0 || desc->n_pages * (int64_t)desc->page_size >= (1ll << 31)) return PDLLM_ERR_SHAPE;
+  if (desc->max_ranges < 0 || desc->max_ranges > pdllm::kMaxRanges) return PDLLM_ERR_UNSUPPORTED;
+  if (table_stride < pdllm::slot_table_stride_for(desc) || ((uintptr_t)table % 4)) return PDLLM_ERR_STRIDE;
+  pdllm::AttnKParams p = {};
+  pdllm::fill_table_params(desc, p);
+  p.slot_stride = table_stride;
+  return pdllm::launch_slot_table(p, desc->n_req, table, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int pdllm_sparse_decode_attn(const pdllm_attn_desc* desc, pdllm_stream_t stream) {
@@ -984,6 +1206,6 @@ extern "C" int pdllm_attn_plan(const pdllm_attn_desc* desc, int32_t prefill, int
   if (st != PDLLM_OK) return st;
   const pdllm::AttnPlan plan = pdllm::make_plan(desc, prefill != 0);
   if (rows_per_group) *rows_per_group = 32 * plan.J;
-  if (num_splits) *num_splits = plan.num_splits;
+  if (num_splits) *num_splits = (plan.t_lin + plan.span - 1) / plan.span;
   return PDLLM_OK;
 }

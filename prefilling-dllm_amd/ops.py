@@ -145,7 +145,8 @@ def load_kvcache(k_cache: torch.Tensor, v_cache: torch.Tensor, context, k_new: t
 # ----------------------------------------------------------------------------------------
 
 def _fill_desc(q, k_new, v_new, out, k_cache, v_cache, block_table, q_start_loc, ranges, mask, mask_mode,
-               max_q_len, max_ctx_len, sm_scale, k_scale, v_scale, num_splits, rows_per_group) -> AttnDesc:
+               max_q_len, max_ctx_len, sm_scale, k_scale, v_scale, num_splits, rows_per_group,
+               tiles_per_workgroup=0) -> AttnDesc:
     n_tokens, Hq, d = q.shape
     Hkv = k_new.shape[1]
     for t in (q, k_new, v_new, out):
@@ -162,6 +163,7 @@ def _fill_desc(q, k_new, v_new, out, k_cache, v_cache, block_table, q_start_loc,
     desc.mask_mode = mask_mode
     desc.sm_scale = float(sm_scale)
     desc.num_splits, desc.rows_per_group = int(num_splits), int(rows_per_group)
+    desc.tiles_per_workgroup = int(tiles_per_workgroup)
     if mask_mode == _lib.MASK_DENSE:
         if mask is None:
             raise ValueError("dense mask mode needs a mask")
@@ -203,7 +205,8 @@ def sparse_decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.T
                             mask_mode: str = "full", mask: Optional[torch.Tensor] = None,
                             sm_scale: Optional[float] = None, k_scale: Optional[torch.Tensor] = None,
                             v_scale: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                            num_splits: int = 0, rows_per_group: int = 0) -> torch.Tensor:
+                            num_splits: int = 0, rows_per_group: int = 0,
+                            tiles_per_workgroup: int = 0) -> torch.Tensor:
     """Attention of the active block over [selected prefix pages || active block].
 
     The visible prefix of request r is either `context_lens[r]` leading tokens of its page
@@ -234,7 +237,8 @@ def sparse_decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.T
         else:
             ranges = tuple(t.to(torch.int32).contiguous() for t in ranges[:3]) + (int(ranges[3]),)
     desc = _fill_desc(q, k_new, v_new, out, k_cache, v_cache, block_table, q_start_loc, ranges, mask, mode,
-                      max_q_len, max_ctx_len, sm_scale, k_scale, v_scale, num_splits, rows_per_group)
+                      max_q_len, max_ctx_len, sm_scale, k_scale, v_scale, num_splits, rows_per_group,
+                      tiles_per_workgroup)
     need = lib.pdllm_attn_workspace_bytes(C.byref(desc))
     if need < 0:
         check(int(need), "sparse_decode_attention")
@@ -252,7 +256,11 @@ class PreparedAttention:
 
     def __init__(self, q, k_new, v_new, k_cache, v_cache, block_table, q_start_loc, *, max_q_len, max_ctx_len,
                  context_lens=None, ranges=None, mask_mode="full", mask=None, sm_scale=None, k_scale=None,
-                 v_scale=None, out=None, num_splits=0, rows_per_group=0, workspace=None):
+                 v_scale=None, out=None, num_splits=0, rows_per_group=0, workspace=None, slot_table=None,
+                 tiles_per_workgroup=0):
+        """slot_table: an int32 tensor from `new_slot_table` shared by every layer of a step; the caller
+        refreshes it with `build_slot_table()` of any one of the prepared layers whenever the page table
+        or the ranges change.  Without it every `run()` rebuilds the table in its workspace."""
         _need_cuda(q, k_new, v_new, q_start_loc)
         n_tokens, Hq, d = q.shape
         self.out = torch.empty_like(q) if out is None else out
@@ -274,7 +282,12 @@ class PreparedAttention:
         self.desc = _fill_desc(q, k_new, v_new, self.out, k_cache, v_cache, block_table, q_start_loc, ranges,
                                mask, mode, max_q_len, max_ctx_len,
                                1.0 / math.sqrt(d) if sm_scale is None else sm_scale, k_scale, v_scale,
-                               num_splits, rows_per_group)
+                               num_splits, rows_per_group, tiles_per_workgroup)
+        self.slot_table = slot_table
+        if slot_table is not None and k_cache is not None and max_ctx_len > 0:
+            if slot_table.dtype != torch.int32 or slot_table.dim() != 2 or slot_table.stride(1) != 1:
+                raise ValueError("slot_table must be an int32 [n_req, stride] tensor (see new_slot_table)")
+            self.desc.slot_table, self.desc.slot_table_stride = slot_table.data_ptr(), slot_table.stride(0)
         need = lib.pdllm_attn_workspace_bytes(C.byref(self.desc))
         if need < 0:
             check(int(need), "PreparedAttention")
@@ -285,7 +298,7 @@ class PreparedAttention:
             self.desc.workspace, self.desc.workspace_bytes = workspace.data_ptr(), int(need)
         # keep every tensor the descriptor points at alive
         self._keep = (q, k_new, v_new, k_cache, v_cache, block_table, q_start_loc, ranges, mask, k_scale, v_scale,
-                      workspace)
+                      workspace, slot_table)
         self._ref = C.byref(self.desc)
         self._fn = lib.pdllm_sparse_decode_attn
 
@@ -294,6 +307,25 @@ class PreparedAttention:
         if st != 0:
             check(st, "PreparedAttention.run")
         return self.out
+
+    def build_slot_table(self, stream: Optional[int] = None) -> None:
+        """(Re)build the shared slot table from this layer's page table and ranges."""
+        if self.slot_table is None:
+            raise ValueError("this PreparedAttention was made without a slot_table")
+        st = lib.pdllm_attn_build_slot_table(self._ref, self.slot_table.data_ptr(), self.slot_table.stride(0),
+                                             torch.cuda.current_stream().cuda_stream if stream is None else stream)
+        if st != 0:
+            check(st, "PreparedAttention.build_slot_table")
+
+
+def new_slot_table(n_req: int, max_ctx_len: int, device) -> torch.Tensor:
+    """An int32 [n_req, stride] tensor of the size pdllm_attn_build_slot_table needs."""
+    desc = AttnDesc()
+    desc.max_ctx_len = int(max_ctx_len)
+    stride = lib.pdllm_attn_slot_table_stride(C.byref(desc))
+    if stride < 0:
+        check(int(stride), "new_slot_table")
+    return torch.zeros((int(n_req), int(stride)), dtype=torch.int32, device=device)
 
 
 def attention_plan(n_req: int, num_q_heads: int, num_kv_heads: int, *, max_q_len: int, max_ctx_len: int,

@@ -18,13 +18,13 @@ def _ops():
 
 
 def run_case(case, dev, *, mask_mode="full", mask=None, rows_per_group=0, num_splits=0, use_ctx_lens=False,
-             sm_scale=None):
+             sm_scale=None, tiles_per_workgroup=0):
     ops = _ops()
     d = lambda t: None if t is None else t.to(dev)
     rp, rs, rl, mr = case.range_tensors()
     kwargs = dict(max_q_len=case.max_q, max_ctx_len=case.max_ctx, mask_mode=mask_mode, mask=d(mask),
                   sm_scale=sm_scale, k_scale=d(case.k_scale), v_scale=d(case.v_scale),
-                  rows_per_group=rows_per_group, num_splits=num_splits)
+                  rows_per_group=rows_per_group, num_splits=num_splits, tiles_per_workgroup=tiles_per_workgroup)
     if use_ctx_lens:
         kwargs["context_lens"] = d(torch.tensor([sum(l for _, l in rr) for rr in case.ranges], dtype=torch.int32))
     else:
@@ -67,6 +67,51 @@ def test_row_group_and_split_variants(dev, rows, splits):
                                        shared_prefix=False)
     ref = oracle_case(case)
     check(run_case(case, dev, rows_per_group=rows, num_splits=splits), ref)
+
+
+@pytest.mark.parametrize("rows", [32, 64, 128, 160])
+@pytest.mark.parametrize("tiles", [1, 2, 3, 5, 7, 100])
+def test_tile_spans_across_columns(dev, rows, tiles):
+    """Workgroups that take a fixed number of tiles of the line of all columns' tiles: pieces of a
+    column end up in different workgroups, one workgroup finishes a column and starts the next, and
+    columns of unequal length (ragged requests) leave empty pieces."""
+    case = configs.chunked_prefix_case(13, n_req=3, n_chunks=5, chunk_tokens=300, topk=2, q_len=40,
+                                       shared_prefix=False)
+    check(run_case(case, dev, rows_per_group=rows, tiles_per_workgroup=tiles), oracle_case(case))
+
+
+def test_tile_spans_causal_dense(dev):
+    case = configs.chunked_prefix_case(17, n_req=2, n_chunks=4, chunk_tokens=200, topk=2, q_len=70,
+                                       shared_prefix=False)
+    check(run_case(case, dev, mask_mode="causal", tiles_per_workgroup=3), oracle_case(case, mask_mode="causal"))
+
+
+def test_shared_slot_table_matches_per_call_table(dev):
+    """A slot table built once (pdllm_attn_build_slot_table) and handed to the prepared descriptor gives
+    the same output as the table the call builds for itself."""
+    ops = _ops()
+    case = configs.chunked_prefix_case(19, n_req=3, n_chunks=6, chunk_tokens=260, topk=3, q_len=48,
+                                       shared_prefix=False)
+    d = lambda t: None if t is None else t.to(dev)
+    rp, rs, rl, mr = case.range_tensors()
+    args = (d(case.q), d(case.k_new), d(case.v_new), d(case.k_cache), d(case.v_cache), d(case.block_table),
+            d(case.q_start_loc))
+    kw = dict(max_q_len=case.max_q, max_ctx_len=case.max_ctx, ranges=(d(rp), d(rs), d(rl), mr))
+    base = ops.sparse_decode_attention(*args, **kw).clone()
+    table = ops.new_slot_table(case.q_start_loc.numel() - 1, case.max_ctx, dev)
+    prep = ops.PreparedAttention(*args, slot_table=table, **kw)
+    prep.build_slot_table()
+    out = prep.run()
+    torch.cuda.synchronize()
+    assert torch.equal(out, base)
+    # the table itself: slot of every visible key, then the count
+    t = table.cpu()
+    for r, rr in enumerate(case.ranges):
+        toks = [s + i for s, l in rr for i in range(l)]
+        assert int(t[r, -1]) == len(toks)
+        bt = case.block_table[r]
+        want = [int(bt[tk // 256]) * 256 + tk % 256 for tk in toks]
+        assert t[r, :len(toks)].tolist() == want
 
 
 @pytest.mark.parametrize("rows", [0, 160, 256])
