@@ -158,6 +158,17 @@ template <int N, typename T>
 __device__ __forceinline__ void lds_wait(T& x) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N) : "memory");
 }
+// the same, and also a fence for three values of the vector pipeline: work that produces them
+// stays before this point, work that consumes them after it (pins the interleaving of softmax
+// arithmetic with the MFMAs, which the compiler would otherwise gather in one place)
+// `keep` is only named as an input: it holds the fragment the MFMA of the step before is still
+// reading, and naming it here keeps the register allocator from handing those registers to the
+// vector instructions in between (a write to a source of a running MFMA stalls the wave until
+// the MFMA has finished, which would serialise the two pipelines).
+template <int N, typename T>
+__device__ __forceinline__ void lds_wait_pin(T& x, float& a, float& b, float& c, const T& keep) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(x), "+v"(a), "+v"(b), "+v"(c) : "n"(N), "v"(keep) : "memory");
+}
 template <int N, typename T>
 __device__ __forceinline__ void lds_wait2(T& x, T& y) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N) : "memory");
@@ -277,6 +288,16 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
       }
     }
   }
+
+  // LDS addresses of this lane's operand fragments in buffer 0 (pipelined loop: the buffer and
+  // key-block offsets are instruction immediates)
+  unsigned ka[8], va[2][4];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) ka[ks] = lds_base + koff[ks];
+#pragma unroll
+  for (int r = 0; r < 2; ++r)
+#pragma unroll
+    for (int db = 0; db < 4; ++db) va[r][db] = lds_base + voff[r][db];
 
   // this workgroup's span of the tile line; it may cover the end of one column and the start of
   // the next, each part ("piece") is an attention pass of its own
@@ -641,6 +662,278 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
     __syncthreads();
   };
 
+  // ------------------------------------------------------------------------------------------
+  // Software-pipelined tile loop (one own row block per wave, bf16 cache).  While the vector
+  // unit turns the scores of tile t into probabilities, the matrix unit already computes the
+  // scores of tile t + 1: each step issues one MFMA of QK(t+1) and the exponentials of two
+  // elements of tile t.  K therefore runs one tile ahead of V in the buffers: iteration t
+  // reads K(t+1) and V(t) and copies K(t+2) and V(t+1).  The last MFMA of a key block writes
+  // into the registers the finished exponentials have just released, so the new scores are in
+  // place for the next iteration without moves.
+  // ------------------------------------------------------------------------------------------
+  constexpr bool PIPELINED = (J == 4) && !KV_FP8;
+  if constexpr (PIPELINED) {
+    if (T0 < T1) {
+      typedef __attribute__((ext_vector_type(8))) short s16x8;
+      int nsv[kDmaGroups];  // slots of the next V tile (nslot holds those of the next K tile)
+      // source of a row = uniform base + 16 B * (slot * row pitch + chunk of this lane)
+      const char* kc_base = static_cast<const char*>(p.k_cache) + (long)kvh * p.cache_head_stride * 2;
+      const char* vc_base = static_cast<const char*>(p.v_cache) + (long)kvh * p.cache_head_stride * 2;
+      const char* kn_base = reinterpret_cast<const char*>(p.k_new + (long)q0 * p.kn_stride + kvh * kD);
+      const char* vn_base = reinterpret_cast<const char*>(p.v_new + (long)q0 * p.vn_stride + kvh * kD);
+      auto issue_k1 = [&](int t, int buf, int i) __attribute__((always_inline)) {
+        const bool ctx = t < Tc;
+        const char* kb = ctx ? kc_base : kn_base;
+        const unsigned kr = ctx ? cache_row16 : kn_row16;
+        char* dst = lds + buf * kBufBytes + wave * 1024;
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(kb + ((unsigned long)((unsigned)nslot[i] * kr + lane_ch) << 4)),
+            (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
+      };
+      auto issue_v1 = [&](int t, int buf, int i) __attribute__((always_inline)) {
+        const bool ctx = t < Tc;
+        const char* vb = ctx ? vc_base : vn_base;
+        const unsigned vr = ctx ? cache_row16 : vn_row16;
+        char* dst = lds + buf * kBufBytes + kTileBytes + wave * 1024;
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(vb + ((unsigned long)((unsigned)nsv[i] * vr + lane_ch) << 4)),
+            (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
+      };
+      auto issue_k = [&](int t, int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kDmaGroups; ++i) issue_k1(t, buf, i);
+      };
+      auto issue_v = [&](int t, int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kDmaGroups; ++i) issue_v1(t, buf, i);
+      };
+      // K fragment read of QK step stp / V^T fragment read of PV step stp; ka and va point into the
+      // buffer in use and move to the other one after every tile
+      auto rdk = [&](bf16x8& dst, int stp) __attribute__((always_inline)) {
+        if ((stp >> 3) == 0) lds_read_b128<0>(dst, ka[stp & 7]);
+        else lds_read_b128<32 * kRowBytes>(dst, ka[stp & 7]);
+      };
+      auto rdv = [&](s16x4& dst, int stp, int r) __attribute__((always_inline)) {
+        constexpr int base = kTileBytes;
+        const int db = stp & 3, kj = stp >> 2;
+        if (kj == 0) lds_read_tr16_b64<base>(dst, va[r][db]);
+        else if (kj == 1) lds_read_tr16_b64<base + 16 * kRowBytes>(dst, va[r][db]);
+        else if (kj == 2) lds_read_tr16_b64<base + 32 * kRowBytes>(dst, va[r][db]);
+        else lds_read_tr16_b64<base + 48 * kRowBytes>(dst, va[r][db]);
+      };
+      constexpr int PF = 3, NS = 16;
+      auto wait_k = [&](bf16x8& x, int stp) __attribute__((always_inline)) {
+        const int young = NS - 1 - stp < PF - 1 ? NS - 1 - stp : PF - 1;
+        if (young == 3) lds_wait<3>(x);
+        else if (young == 2) lds_wait<2>(x);
+        else if (young == 1) lds_wait<1>(x);
+        else lds_wait<0>(x);
+      };
+
+      // one iteration: softmax of tile t (scores in Sc) interleaved with QK of tile t + 1 (into Sn),
+      // then PV of tile t.  PAR = buffer of V(t); K(t+1) sits in the other buffer.
+      int flip = kBufBytes;  // ka: buffer 1 -> 0 -> 1 ..., va: buffer 0 -> 1 -> 0 ...
+      auto iter = [&](int t, int PAR, f32x16 (&Sc)[2]) __attribute__((always_inline)) {
+        const bool has_next = t + 1 < T1;
+        // The copies of V(t+1) (slots in nsv) and K(t+2) (slots in nslot) are handed out one per
+        // second step of the QK loop below: a burst would block the wave on the memory pipeline.
+        const bool k_on = t + 2 < T1;
+        if (has_next) build_mask(t + 1, PAR ^ 1);
+
+        const bool active = t >= Tc;
+        const int a0 = active ? (t - Tc) * kKT : 0;
+        int nvalid = active ? Sa - a0 : ctx_total - t * kKT;
+        const bool generic = nvalid < kKT || (active && p.mask_mode != PDLLM_MASK_FULL);
+        nvalid = nvalid < kKT ? nvalid : kKT;
+        // ---- masks, row maximum, lazy rescale (vector unit only) ----
+        if (generic) {
+          int lim = nvalid;
+          if (active && p.mask_mode == PDLLM_MASK_CAUSAL) { const int cl = srowA - a0 + 1; lim = cl < lim ? cl : lim; }
+          int tl = srowA - tq_first;
+          tl = tl < 0 ? 0 : (tl >= kMaxTok ? kMaxTok - 1 : tl);
+          const uint32_t* mrow = (active && p.mask_mode == PDLLM_MASK_DENSE) ? &s_maskbits[PAR][tl][0] : nullptr;
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            const int lb = lim - 32 * b;
+            uint32_t W = lb >= 32 ? 0xffffffffu : (lb <= 0 ? 0u : ((1u << lb) - 1u));
+            if (mrow != nullptr) W &= mrow[b];
+            W >>= 4 * h;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              constexpr uint32_t one = 1u;
+              const uint32_t bit = one << (8 * (i >> 2) + (i & 3));
+              Sc[b][i] = (W & bit) ? Sc[b][i] : -INFINITY;
+            }
+          }
+        }
+        float mx = fmaxf(Sc[0][0], Sc[0][1]);
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int i = (b == 0 ? 2 : 0); i < 16; i += 2) mx = fmaxf(fmaxf(mx, Sc[b][i]), Sc[b][i + 1]);
+        mx = half_swap_max(mx);
+        const bool need = mx > kRescaleSlack || (MA == -INFINITY && mx > -INFINITY);
+        if (__builtin_amdgcn_ballot_w64(need) != 0) {
+          const float Muse = (MA == -INFINITY) ? 0.f : MA;
+          const float Mn = fmaxf(MA, Muse + mx);
+          const float alpha = (Mn == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(MA - Mn);
+          const float delta = ((Mn == -INFINITY) ? 0.f : Mn) - Muse;
+          MA = Mn;
+          lA *= alpha;
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) Sc[b][i] -= delta;
+#pragma unroll
+          for (int db = 0; db < 4; ++db) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) OA[db][i] *= alpha;
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+        // ---- exponentials of tile t, two per step, between the MFMAs of QK(t+1) ----
+        const float init = (MA == -INFINITY) ? 0.f : -MA;
+        f32x16 Sn[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) Sn[b][i] = init;
+        bf16x8 P[2][2];
+        const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
+        float psum = 0.f;
+        auto exp_pair = [&](int stp) __attribute__((always_inline)) {
+          const int b = stp >> 3, i = 2 * (stp & 7);
+          const bf16x2 pr = {(__bf16)__builtin_amdgcn_exp2f(Sc[b][i]), (__bf16)__builtin_amdgcn_exp2f(Sc[b][i + 1])};
+          psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);
+          P[b][i >> 3][i & 7] = pr[0];
+          P[b][i >> 3][(i & 7) + 1] = pr[1];
+        };
+        if (has_next) {
+          bf16x8 kf[PF];
+#pragma unroll
+          for (int i = 0; i < PF; ++i) rdk(kf[i], i);
+          bf16x8 used = kf[0];  // fragment of the MFMA issued in the step before
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int stp = 0; stp < NS; ++stp) {
+            {
+              // wait for this step's K fragment; the step's two scores enter and the running sum of
+              // the step before leaves through the same statement
+              float e0 = Sc[stp >> 3][2 * (stp & 7)];
+              float e1 = Sc[stp >> 3][2 * (stp & 7) + 1];
+              const int young = NS - 1 - stp < PF - 1 ? NS - 1 - stp : PF - 1;
+              if (young == 3) lds_wait_pin<3>(kf[stp % PF], e0, e1, psum, used);
+              else if (young == 2) lds_wait_pin<2>(kf[stp % PF], e0, e1, psum, used);
+              else if (young == 1) lds_wait_pin<1>(kf[stp % PF], e0, e1, psum, used);
+              else lds_wait_pin<0>(kf[stp % PF], e0, e1, psum, used);
+              used = kf[stp % PF];
+              Sc[stp >> 3][2 * (stp & 7)] = e0;
+              Sc[stp >> 3][2 * (stp & 7) + 1] = e1;
+            }
+            if ((stp & 7) == 7) {
+              // the block's exponentials are all issued: its registers take the finished scores
+              exp_pair(stp);
+              Sc[stp >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], QA[7], Sn[stp >> 3], 0, 0, 0);
+            } else {
+              Sn[stp >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], QA[stp & 7], Sn[stp >> 3], 0, 0, 0);
+              exp_pair(stp);
+            }
+            if (stp + PF < NS) rdk(kf[stp % PF], stp + PF);
+            if ((stp & 1) == 1) {
+              if (stp < 8) issue_v1(t + 1, PAR ^ 1, stp >> 1);
+              else if (k_on) issue_k1(t + 2, PAR, (stp >> 1) - 4);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+#pragma unroll
+          for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
+          if (t + 3 < T1) load_slots(t + 3);
+        } else {
+#pragma unroll
+          for (int stp = 0; stp < NS; ++stp) exp_pair(stp);
+        }
+        lA += psum;
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- PV of tile t ----
+        {
+          s16x4 lo[2], hi[2];
+          rdv(lo[0], 0, 0); rdv(hi[0], 0, 1);
+          rdv(lo[1], 1, 0); rdv(hi[1], 1, 1);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int stp = 0; stp < NS; ++stp) {
+            const int db = stp & 3, kj = stp >> 2;
+            if (stp + 1 < NS) lds_wait2<2>(lo[stp & 1], hi[stp & 1]);
+            else lds_wait2<0>(lo[stp & 1], hi[stp & 1]);
+            const s16x4 a = lo[stp & 1], b2 = hi[stp & 1];
+            const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
+            OA[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), P[kj >> 1][kj & 1], OA[db], 0, 0, 0);
+            if (stp + 2 < NS) { rdv(lo[stp & 1], stp + 2, 0); rdv(hi[stp & 1], stp + 2, 1); }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+        // the next tile reads the other buffers
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) ka[ks] -= flip;
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+          for (int db = 0; db < 4; ++db) va[r][db] += flip;
+        flip = -flip;
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): K(t+2), V(t+1) and the slots have landed
+        __syncthreads();
+      };
+
+      // ---- prologue: K(T0), V(T0); then K(T0+1) while QK(T0) runs unpipelined ----
+      f32x16 SX[2];
+      load_slots(T0);
+#pragma unroll
+      for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
+      issue_k(T0, 0);
+      issue_v(T0, 0);
+      if (T0 + 1 < T1) load_slots(T0 + 1);
+      build_mask(T0, 0);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+      if (T0 + 1 < T1) issue_k(T0 + 1, 1);
+#pragma unroll
+      for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
+      if (T0 + 2 < T1) load_slots(T0 + 2);
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) SX[b][i] = 0.f;
+      {
+        bf16x8 kf[PF];
+#pragma unroll
+        for (int i = 0; i < PF; ++i) rdk(kf[i], i);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int stp = 0; stp < NS; ++stp) {
+          wait_k(kf[stp % PF], stp);
+          SX[stp >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], QA[stp & 7], SX[stp >> 3], 0, 0, 0);
+          if (stp + PF < NS) rdk(kf[stp % PF], stp + PF);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      // from here on ka reads K(t+1) in buffer 1 and va reads V(t) in buffer 0
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) ka[ks] += kBufBytes;
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+      for (int t = T0; t < T1; ++t) iter(t, (t - T0) & 1, SX);
+      // leave ka / va pointing at buffer 0 for the next piece
+      if (flip > 0) {
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) ka[ks] -= kBufBytes;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+          for (int db = 0; db < 4; ++db) va[r][db] -= kBufBytes;
+      }
+    }
+  } else
   if (T0 < T1) {
     load_slots(T0);
     issue_tile(T0, 0);  // waits for the slots it uses
