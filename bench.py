@@ -128,6 +128,120 @@ def cpu_baseline(torch, w, sample_layers=1):
     return per_layer, cores, ref
 
 
+def _time_us(torch, fn, iters=10, warmup=2):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / iters
+
+
+def secondary_shapes(torch, ops, dev):
+    """The other BASELINE configs, one launch (or one layer) each: reported next to the headline number."""
+    out = {}
+    gd = torch.Generator(device=dev).manual_seed(1)
+    std = 1.0 / math.sqrt(D)
+
+    # response-only block (the reference engine's real decode shape, 32 rows): the HBM-bound case
+    w32 = build_workload(torch, dev, q_len=32, layers=4)
+    p32 = prepare(ops, w32)
+    _, g32 = time_steps(torch, p32, 16, 2)
+    b32, f32_ = algorithmic_work(32, w32["ctx"], w32["n_req"])
+    l32 = g32 / (16 * 4)
+    out["decode_32_rows"] = {"us_per_launch": l32 * 1e6, "us_per_step_28_layers": l32 * 28e6,
+                             "hbm_GBps": b32 / l32 / 1e9, "hbm_frac": b32 / l32 / 1e9 / PEAK_HBM_GBS,
+                             "bf16_TFLOPs": f32_ / l32 / 1e12}
+    del w32, p32
+
+    # configs[3]: chunked BOS-prefixed prefill, 32 chunks x 1025 rows, causal inside a chunk, with the paged
+    # store of K/V (one layer; a prefill is 28 of these)
+    L, NC = 1025, 32
+    n = L * NC
+    q = (torch.randn((n, HQ, D), generator=gd, device=dev) * std).to(torch.bfloat16)
+    k = (torch.randn((n, HKV, D), generator=gd, device=dev) * std).to(torch.bfloat16)
+    v = (torch.randn((n, HKV, D), generator=gd, device=dev) * std).to(torch.bfloat16)
+    o = torch.empty_like(q)
+    pages = (n + PAGE - 1) // PAGE
+    kc = torch.zeros((pages + 1, PAGE, HKV, D), dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    page_ids = torch.randperm(pages, generator=torch.Generator().manual_seed(2)).to(torch.int32).to(dev)
+    slots = ops.slot_mapping_from_pages(page_ids, n)
+    cu = torch.arange(0, n + 1, L, dtype=torch.int32, device=dev)
+    us = _time_us(torch, lambda: ops.chunk_prefill_attention(q, k, v, cu, max_seqlen=L, causal=True, k_cache=kc,
+                                                             v_cache=vc, slot_mapping=slots, out=o), 5, 1)
+    fl = 2.0 * NC * L * L * D * HQ
+    out["prefill_32x1025_causal_layer"] = {"us_per_layer": us, "bf16_TFLOPs": fl / us / 1e6,
+                                           "mfma_frac": fl / us / 1e6 / PEAK_BF16_TFLOPS,
+                                           "us_per_prefill_28_layers": us * 28}
+    del q, k, v, o, kc, vc
+
+    # configs[1]: draft self-information scores of 32 chunks x 4 labels over a 152064 vocabulary + top-4,
+    # and the column-sum eviction scores of 8 chunks (28 heads x 64 queries x 1025 keys fp32) + keep 256
+    V2 = 152064
+    logits = (torch.randn((32, 4, V2), generator=gd, device=dev) * 2.0).to(torch.bfloat16)
+    labels = torch.randint(0, V2, (32, 4), generator=gd, device=dev)
+    us = _time_us(torch, lambda: ops.topk_lowest_index(ops.chunk_scores_from_logits(logits, labels), 4))
+    by = logits.numel() * 2
+    out["score_32x4x152064_top4"] = {"us": us, "hbm_GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS}
+    probs = torch.softmax(torch.randn((8, HQ, 64, 1025), generator=gd, device=dev), dim=-1)
+    us = _time_us(torch, lambda: ops.topb_keep_bos(ops.evict_colsum(probs).reshape(8, 1025), 256))
+    by = probs.numel() * 4
+    out["evict_8x28x64x1025_keep256"] = {"us": us, "hbm_GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS}
+    del logits, probs
+
+    # configs[4]: confidence + argmax over [4 x 32, 126464] logits and the threshold-0.9 unmask decision
+    V5 = 126464
+    lg = (torch.randn((128, V5), generator=gd, device=dev) * 3.0).to(torch.bfloat16)
+    ids = torch.full((4, 32), V5 - 1, dtype=torch.int64, device=dev)
+
+    def unmask():
+        conf, tok = ops.conf_argmax(lg, 32)
+        ids.fill_(V5 - 1)
+        ops.threshold_unmask(conf, tok, ids, V5 - 1, 0.9)
+    us = _time_us(torch, unmask)
+    by = lg.numel() * 2
+    out["unmask_4x32x126464"] = {"us": us, "hbm_GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS}
+    del lg
+
+    # configs[4]: fp8 e4m3 KV pages with a per-page scale, MHA 32/32, 4 requests x 16 chunks x 1025 tokens, 160 rows
+    Hm, n_req, ctx5, ql = 32, 4, 16 * 1025, 160
+    ppr = 64 * 1025 // PAGE + 1
+    n_pages = n_req * ppr + 1
+    kc8 = torch.randint(0, 0x78, (n_pages, PAGE, Hm, D), dtype=torch.uint8, device=dev, generator=gd)
+    vc8 = torch.randint(0, 0x78, (n_pages, PAGE, Hm, D), dtype=torch.uint8, device=dev, generator=gd)
+    ks = torch.full((n_pages,), 1.0 / 448, dtype=torch.float32, device=dev)
+    vs = torch.full((n_pages,), 1.0 / 448, dtype=torch.float32, device=dev)
+    bt = torch.arange(n_req * ppr, dtype=torch.int32, device=dev).view(n_req, ppr)
+    g = torch.Generator().manual_seed(3)
+    ptr, start, length = [0], [], []
+    for r in range(n_req):
+        for c in sorted(torch.randperm(64, generator=g)[:16].tolist()):
+            start.append(c * 1025)
+            length.append(1025)
+        ptr.append(len(start))
+    mk = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    q5 = (torch.randn((n_req * ql, Hm, D), generator=gd, device=dev) * std).to(torch.bfloat16)
+    k5 = (torch.randn((n_req * ql, Hm, D), generator=gd, device=dev) * std).to(torch.bfloat16)
+    v5 = (torch.randn((n_req * ql, Hm, D), generator=gd, device=dev) * std).to(torch.bfloat16)
+    qsl = torch.arange(0, n_req * ql + 1, ql, dtype=torch.int32, device=dev)
+    table = ops.new_slot_table(n_req, ctx5, dev)
+    pr = ops.PreparedAttention(q5, k5, v5, kc8, vc8, bt, qsl, max_q_len=ql, max_ctx_len=ctx5,
+                               ranges=(mk(ptr), mk(start), mk(length), 16), k_scale=ks, v_scale=vs, slot_table=table)
+    pr.build_slot_table()
+    us = _time_us(torch, pr.run, 5, 1)
+    by = n_req * (2 * ctx5 * Hm * D * 1 + 2 * ql * Hm * D * 2 + 2 * ql * Hm * D * 2)
+    fl = n_req * 4.0 * ql * (ctx5 + ql) * D * Hm
+    out["decode_fp8_kv_4x16x1025_mha32_layer"] = {"us_per_layer": us, "hbm_GBps": by / us / 1e3,
+                                                  "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS,
+                                                  "bf16_TFLOPs": fl / us / 1e6}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -186,18 +300,7 @@ def main():
                "sample": f"1 of {w['layers']} layers x {w['n_req']} requests of the same step (median of 3), "
                          f"extrapolated x{w['layers']}", "max_abs_err_vs_gpu": err}
 
-    extras = {}
-    if not args.no_extras:
-        # response-only block (the reference engine's real decode shape, 32 rows): the HBM-bound case
-        w32 = build_workload(torch, dev, q_len=32, layers=4)
-        p32 = prepare(ops, w32)
-        _, g32 = time_steps(torch, p32, 16, 2)
-        b32, f32_ = algorithmic_work(32, w32["ctx"], w32["n_req"])
-        l32 = g32 / (16 * 4)
-        extras["decode_32_rows"] = {"us_per_launch": l32 * 1e6, "us_per_step_28_layers": l32 * 28e6,
-                                    "hbm_GBps": b32 / l32 / 1e9, "hbm_frac": b32 / l32 / 1e9 / PEAK_HBM_GBS,
-                                    "bf16_TFLOPs": f32_ / l32 / 1e12}
-        del w32, p32
+    extras = secondary_shapes(torch, ops, dev) if not args.no_extras else {}
 
     rows, splits = ops.attention_plan(w["n_req"], HQ, HKV, max_q_len=w["q_len"], max_ctx_len=w["ctx"],
                                       num_splits=args.num_splits, rows_per_group=args.rows_per_group)

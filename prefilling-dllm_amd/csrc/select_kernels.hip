@@ -98,6 +98,7 @@ __global__ __launch_bounds__(256) void topk_sort_kernel(const float* __restrict_
 
 // Radix select for long rows (n up to 65536): finds the k-th best 32-bit key, then keeps all
 // better keys and the lowest-index ties.  Output ascending by index.  One workgroup per row.
+template <bool CACHED>  // CACHED: n <= 2048, every thread keeps the keys of its span in registers
 __global__ __launch_bounds__(256) void topk_radix_kernel(const float* __restrict__ scores, long n,
                                                          long stride, long k, int descending,
                                                          int force_first, int nonfinite_to_neginf,
@@ -108,6 +109,7 @@ __global__ __launch_bounds__(256) void topk_radix_kernel(const float* __restrict
   __shared__ int wave_tot[4][2];
   const long row = blockIdx.x;
   const float* s = scores + row * stride;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   auto key_of = [&](long i) -> uint32_t {
     float v = s[i];
     if (nonfinite_to_neginf && !(fabsf(v) <= 3.402823466e38f)) v = -INFINITY;
@@ -118,6 +120,16 @@ __global__ __launch_bounds__(256) void topk_radix_kernel(const float* __restrict
   };
   // note: with force_first the forced element shares key 0 only with scores that map to 0,
   // i.e. +NaN in descending order; index order still puts position 0 first.
+  // Every thread owns a contiguous span of indices (the output is in index order).
+  const long span = CACHED ? 8 : (n + 255) / 256;
+  const long begin = threadIdx.x * span;
+  long end = begin + span;
+  end = end < n ? end : n;
+  uint32_t ck[8];
+  if (CACHED) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) ck[u] = begin + u < n ? key_of(begin + u) : 0xffffffffu;
+  }
   if (threadIdx.x == 0) { s_prefix = 0u; s_need = (int)k; }
   __syncthreads();
   for (int pass = 0; pass < 4; ++pass) {
@@ -125,37 +137,50 @@ __global__ __launch_bounds__(256) void topk_radix_kernel(const float* __restrict
     hist[threadIdx.x] = 0;
     __syncthreads();
     const uint32_t prefix = s_prefix;
+    const int need = s_need;
     const uint32_t pmask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
-    for (long i = threadIdx.x; i < n; i += 256) {
-      const uint32_t kk = key_of(i);
-      if ((kk & pmask) == prefix) atomicAdd(&hist[(kk >> shift) & 255], 1);
+    if (CACHED) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (begin + u < n && (ck[u] & pmask) == prefix) atomicAdd(&hist[(ck[u] >> shift) & 255], 1);
+    } else {
+      for (long i = threadIdx.x; i < n; i += 256) {
+        const uint32_t kk = key_of(i);
+        if ((kk & pmask) == prefix) atomicAdd(&hist[(kk >> shift) & 255], 1);
+      }
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      int need = s_need, b = 0;
-      for (; b < 256; ++b) {
-        if (hist[b] >= need) break;
-        need -= hist[b];
-      }
-      s_need = need;
-      s_prefix = prefix | ((uint32_t)b << shift);
+    // the bin that holds the need-th smallest key: inclusive scan of the 256 bins, one per thread
+    const int mine = hist[threadIdx.x];
+    int incl = mine;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int v = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += v;
+    }
+    if (lane == 63) wave_tot[wave][0] = incl;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) incl += wave_tot[w][0];
+    if (incl >= need && incl - mine < need) {  // exactly one thread
+      s_need = need - (incl - mine);
+      s_prefix = prefix | ((uint32_t)threadIdx.x << shift);
     }
     __syncthreads();
   }
   const uint32_t kth = s_prefix;  // key of the k-th best element
   const int need_eq = s_need;     // how many elements equal to kth are kept (lowest indices)
-  // ordered compaction: thread owns a contiguous span of indices
-  const long span = (n + 255) / 256;
-  const long begin = threadIdx.x * span;
-  long end = begin + span;
-  end = end < n ? end : n;
   int c_lt = 0, c_eq = 0;
-  for (long i = begin; i < end; ++i) {
-    const uint32_t kk = key_of(i);
-    c_lt += kk < kth;
-    c_eq += kk == kth;
+  if (CACHED) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (begin + u < n) { c_lt += ck[u] < kth; c_eq += ck[u] == kth; }
+  } else {
+    for (long i = begin; i < end; ++i) {
+      const uint32_t kk = key_of(i);
+      c_lt += kk < kth;
+      c_eq += kk == kth;
+    }
   }
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int i_lt = c_lt, i_eq = c_eq;
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
@@ -167,8 +192,7 @@ __global__ __launch_bounds__(256) void topk_radix_kernel(const float* __restrict
   int b_lt = i_lt - c_lt, b_eq = i_eq - c_eq;
   for (int w = 0; w < wave; ++w) { b_lt += wave_tot[w][0]; b_eq += wave_tot[w][1]; }
   // position in the output = (#kept with lower index)
-  for (long i = begin; i < end; ++i) {
-    const uint32_t kk = key_of(i);
+  auto place = [&](long i, uint32_t kk) {
     const int eq_kept_before = b_eq < need_eq ? b_eq : need_eq;
     if (kk < kth) {
       out[row * k + b_lt + eq_kept_before] = i;
@@ -177,6 +201,13 @@ __global__ __launch_bounds__(256) void topk_radix_kernel(const float* __restrict
       if (b_eq < need_eq) out[row * k + b_lt + b_eq] = i;
       ++b_eq;
     }
+  };
+  if (CACHED) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (begin + u < n) place(begin + u, ck[u]);
+  } else {
+    for (long i = begin; i < end; ++i) place(i, key_of(i));
   }
 }
 
@@ -184,37 +215,43 @@ __global__ __launch_bounds__(256) void topk_radix_kernel(const float* __restrict
 // column sums of probabilities: out[c, g, k] = sum_{h in group g} ( sum_q p[c, h, q, k] )
 // inner sums run over q in index order, then heads in index order (fixed, reproducible).
 // ---------------------------------------------------------------------------------------
-constexpr int kColBlock = 64;
-
+// One workgroup = (chunk, block of CB key columns).  Its 256 threads form 256/CB head slots x CB
+// columns; a thread adds the query rows of a head in index order for its column (a row of CB columns is
+// one contiguous segment), then the heads of a group are added in index order from LDS.  The summation
+// order depends on nothing but the indices, so the result is reproducible bit for bit.  Narrow column
+// blocks are used when there are few chunks, so that the grid still fills the chip.
+template <int CB>
 __global__ __launch_bounds__(256) void evict_colsum_kernel(const float* __restrict__ probs, long n_heads,
                                                            long n_q, long n_keys, long hpg,
                                                            float* __restrict__ out) {
-  extern __shared__ float head_sum[];  // [n_heads][kColBlock]
+  constexpr int NH = 256 / CB;
+  extern __shared__ float head_sum[];  // [n_heads][CB]
   const long chunk = blockIdx.y;
-  const long col = (long)blockIdx.x * kColBlock + (threadIdx.x & 63);
-  const int sub = threadIdx.x >> 6;
+  const int c = threadIdx.x % CB;
+  const int sub = threadIdx.x / CB;
+  const long col = (long)blockIdx.x * CB + c;
   const float* base = probs + chunk * n_heads * n_q * n_keys;
-  for (long hd = sub; hd < n_heads; hd += 4) {
+  for (long hd = sub; hd < n_heads; hd += NH) {
     float acc = 0.f;
     if (col < n_keys) {
       const float* p = base + hd * n_q * n_keys + col;
       long q = 0;
-      for (; q + 8 <= n_q; q += 8) {
-        float v[8];
+      for (; q + 16 <= n_q; q += 16) {
+        float v[16];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = p[(q + u) * n_keys];
+        for (int u = 0; u < 16; ++u) v[u] = p[(q + u) * n_keys];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) acc += v[u];
+        for (int u = 0; u < 16; ++u) acc += v[u];
       }
       for (; q < n_q; ++q) acc += p[q * n_keys];
     }
-    head_sum[hd * kColBlock + (threadIdx.x & 63)] = acc;
+    head_sum[hd * CB + c] = acc;
   }
   __syncthreads();
   const long n_groups = n_heads / hpg;
-  for (long g = sub; g < n_groups; g += 4) {
+  for (long g = sub; g < n_groups; g += NH) {
     float acc = 0.f;
-    for (long hh = 0; hh < hpg; ++hh) acc += head_sum[(g * hpg + hh) * kColBlock + (threadIdx.x & 63)];
+    for (long hh = 0; hh < hpg; ++hh) acc += head_sum[(g * hpg + hh) * CB + c];
     if (col < n_keys) out[(chunk * n_groups + g) * n_keys + col] = acc;
   }
 }
@@ -335,15 +372,19 @@ static int topk_launch(const float* scores, int64_t n_rows, int64_t n, int64_t s
   if (n_rows < 0 || n <= 0 || k < 0 || k > n || stride < n || n > 65536) return PDLLM_ERR_SHAPE;
   if (n_rows == 0 || k == 0) return PDLLM_OK;
   if (n_rows > 0x7fffffffL) return PDLLM_ERR_SHAPE;
-  if (n <= kSortMax) {
+  // an ascending index set only needs the k-th key (radix select); the full sort is for rank order
+  if (n <= kSortMax && (!sorted_ascending || n <= 256)) {
     hipLaunchKernelGGL(topk_sort_kernel, dim3((unsigned)n_rows), dim3(256), 0, stream, scores, (long)n,
                        (long)stride, (long)k, descending, force_first, nonfinite, sorted_ascending,
                        reinterpret_cast<long*>(out));
   } else {
     if (!sorted_ascending) return PDLLM_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(topk_radix_kernel, dim3((unsigned)n_rows), dim3(256), 0, stream, scores, (long)n,
-                       (long)stride, (long)k, descending, force_first, nonfinite,
-                       reinterpret_cast<long*>(out));
+    if (n <= 2048)
+      hipLaunchKernelGGL(topk_radix_kernel<true>, dim3((unsigned)n_rows), dim3(256), 0, stream, scores, (long)n,
+                         (long)stride, (long)k, descending, force_first, nonfinite, reinterpret_cast<long*>(out));
+    else
+      hipLaunchKernelGGL(topk_radix_kernel<false>, dim3((unsigned)n_rows), dim3(256), 0, stream, scores, (long)n,
+                         (long)stride, (long)k, descending, force_first, nonfinite, reinterpret_cast<long*>(out));
   }
   return launch_status();
 }
@@ -378,11 +419,20 @@ extern "C" int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t 
       n_heads % heads_per_group)
     return PDLLM_ERR_SHAPE;
   if (n_chunks == 0) return PDLLM_OK;
-  if (n_chunks > 65535 || n_heads * kColBlock * 4 > 64 * 1024) return PDLLM_ERR_UNSUPPORTED;
-  const dim3 grid((unsigned)((n_keys + kColBlock - 1) / kColBlock), (unsigned)n_chunks);
-  hipLaunchKernelGGL(evict_colsum_kernel, grid, dim3(256), (size_t)(n_heads * kColBlock * 4),
-                     static_cast<hipStream_t>(stream), probs, (long)n_heads, (long)n_queries, (long)n_keys,
-                     (long)heads_per_group, scores_out);
+  if (n_chunks > 65535 || n_heads * 64 * 4 > 64 * 1024) return PDLLM_ERR_UNSUPPORTED;
+  const size_t lds = (size_t)(n_heads * 64 * 4);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const long blocks64 = (n_keys + 63) / 64 * n_chunks;
+  if (blocks64 >= 1024) {
+    hipLaunchKernelGGL(evict_colsum_kernel<64>, dim3((unsigned)((n_keys + 63) / 64), (unsigned)n_chunks), dim3(256),
+                       lds, st, probs, (long)n_heads, (long)n_queries, (long)n_keys, (long)heads_per_group, scores_out);
+  } else if (blocks64 >= 128) {
+    hipLaunchKernelGGL(evict_colsum_kernel<32>, dim3((unsigned)((n_keys + 31) / 32), (unsigned)n_chunks), dim3(256),
+                       lds, st, probs, (long)n_heads, (long)n_queries, (long)n_keys, (long)heads_per_group, scores_out);
+  } else {
+    hipLaunchKernelGGL(evict_colsum_kernel<16>, dim3((unsigned)((n_keys + 15) / 16), (unsigned)n_chunks), dim3(256),
+                       lds, st, probs, (long)n_heads, (long)n_queries, (long)n_keys, (long)heads_per_group, scores_out);
+  }
   return launch_status();
 }
 
