@@ -13,7 +13,7 @@
 //   With J >= 4 wave w owns row block w ("slot A") for all keys.  The remaining blocks
 //   ("slot B") are shared: J=6 -> blocks 4,5, each split between two waves that take one
 //   32-key block of every tile; J=5 -> block 4 split over all four waves, two of them on even
-//   tiles and two on odd tiles; J=8 -> a second full block per wave.  J=1,2 have only shared
+//   tiles and two on odd tiles; J=8 -> a workgroup of 8 wavefronts, one block each.  J=1,2 have only shared
 //   blocks (intra-workgroup split-KV for short active blocks).  Shared blocks are merged
 //   through LDS with a log-sum-exp reduction.  An optional split over workgroups writes fp32
 //   partials + LSE to a workspace that attn_merge_kernel reduces.
@@ -51,12 +51,11 @@ typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 constexpr int kD = 128;          // head dim
 constexpr int kKT = 64;          // keys per tile
 constexpr int kNKB = kKT / 32;   // 32-key blocks per tile
-constexpr int kThreads = 256;    // 4 wavefronts
+constexpr int kThreads = 256;    // 4 wavefronts (8 for the 256-row group)
 constexpr int kRowBytes = 256;   // one K or V row in LDS
 constexpr int kTileBytes = kKT * kRowBytes;      // 16384
 constexpr int kBufBytes = 2 * kTileBytes;        // K tile + V tile
 constexpr int kMainBytes = 2 * kBufBytes;        // double buffered: 65536
-constexpr int kDmaGroups = kKT / 16;             // 16-row groups of a tile; a wave copies 4 rows of each
 constexpr int kPartBytes = kD * 32 * 4;          // LDS partial of a shared row block: [d][row ^ (d & 31)] fp32
 constexpr int kMaxRanges = 128;
 constexpr int kMaxTok = 264;                     // query tokens a row group of 256 rows can touch (+ slack)
@@ -246,10 +245,12 @@ __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB
 }
 
 template <int KV_FP8, int J>
-__global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd_kernel(const AttnKParams p) {
+__global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_kernel(const AttnKParams p) {
+  constexpr int NW = J == 8 ? 8 : 4;        // wavefronts per workgroup
+  constexpr int kDmaGroups = 16 / NW;       // a tile is 16 groups of 4 rows; a wave copies this many of them
   constexpr bool HAS_A = J >= 4;
-  constexpr bool DUAL = J == 8;                                  // slot B = a second full block per wave
-  constexpr bool HAS_B = J != 4;
+  constexpr bool DUAL = false;
+  constexpr bool HAS_B = J != 4 && J != 8;
   constexpr int GS = (J == 1 || J == 5) ? 4 : (J == 2 || J == 6) ? 2 : 1;  // waves sharing a B block
   constexpr bool QB_LDS = J == 5 || J == 6;  // Q of the shared block(s) lives in LDS, not in registers
 
@@ -355,7 +356,6 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
   else if (J == 2) blkB = wave >> 1;
   else if (J == 5) blkB = 4;
   else if (J == 6) blkB = 4 + (wave >> 1);
-  else if (J == 8) blkB = 4 + wave;
   const int kbB = gi & 1;       // key block of a tile this wave handles for a shared block
   const int parB = (gi >> 1) ^ (row_tile & 1);  // GS == 4: tiles of this parity only
 
@@ -409,7 +409,7 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
   auto build_mask = [&](int t, int par) __attribute__((always_inline)) {
     if (p.mask_mode != PDLLM_MASK_DENSE || t < Tc) return;
     const int a0 = (t - Tc) * kKT;
-    for (int idx = tid; idx < ntok * kNKB; idx += kThreads) {
+    for (int idx = tid; idx < ntok * kNKB; idx += NW * 64) {
       const int tok = idx / kNKB, w = idx % kNKB;
       const uint8_t* mp = mask_base + (long)(tq_first + tok) * p.mask_stride + a0 + 32 * w;
       uint32_t bits = 0;
@@ -423,8 +423,8 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
   uint2 st_k[kDmaGroups], st_v[kDmaGroups];
   float st_ks[kDmaGroups], st_vs[kDmaGroups];
 
-  // Copy of tile t into buffer `buf`: this wave moves rows 16*i + 4*wave + lane/16 for each 16-row
-  // group i, one instruction for K and one for V.  The chunk a lane fetches,
+  // Copy of tile t into buffer `buf`: this wave moves rows 4*NW*i + 4*wave + lane/16 for
+  // i < kDmaGroups, one instruction for K and one for V each.  The chunk a lane fetches,
   // (lane & 15) ^ swz(row), does not depend on i because the swizzle has period 16.
   // The source rows are cache slots read from the slot table (prefix tiles) or rows of the
   // active block; they are fetched into registers one tile before the copy is issued.
@@ -442,12 +442,12 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
   auto load_slots = [&](int t) __attribute__((always_inline)) {
     if (t < Tc) {
 #pragma unroll
-      for (int i = 0; i < kDmaGroups; ++i) nslot[i] = tbl[t * kKT + 16 * i + lane_row];
+      for (int i = 0; i < kDmaGroups; ++i) nslot[i] = tbl[t * kKT + 4 * NW * i + lane_row];
     } else {
       const int a0 = (t - Tc) * kKT;
 #pragma unroll
       for (int i = 0; i < kDmaGroups; ++i) {
-        const int a = a0 + 16 * i + lane_row;
+        const int a = a0 + 4 * NW * i + lane_row;
         nslot[i] = a < Sa ? a : a0;  // padding rows copy the first (always valid) row; they are masked
       }
     }
@@ -475,10 +475,10 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
       for (int i = 0; i < kDmaGroups; ++i) {
         __builtin_amdgcn_global_load_lds(
             (const __attribute__((address_space(1))) void*)(kb + ((unsigned long)((unsigned)nslot[i] * kr) << 4)),
-            (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
+            (__attribute__((address_space(3))) void*)(dst + i * (NW * 1024)), 16, 0, 0);
         __builtin_amdgcn_global_load_lds(
             (const __attribute__((address_space(1))) void*)(vb + ((unsigned long)((unsigned)nslot[i] * vr) << 4)),
-            (__attribute__((address_space(3))) void*)(dst + i * 4096 + kTileBytes), 16, 0, 0);
+            (__attribute__((address_space(3))) void*)(dst + i * (NW * 1024) + kTileBytes), 16, 0, 0);
       }
     }
   };
@@ -487,7 +487,7 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
     if (KV_FP8 && t < Tc) {
 #pragma unroll
       for (int i = 0; i < kDmaGroups; ++i) {
-        char* kdst = lds + buf * kBufBytes + (i * 4 + wave) * 1024 + lane * 16;
+        char* kdst = lds + buf * kBufBytes + (i * NW + wave) * 1024 + lane * 16;
         *reinterpret_cast<uint4*>(kdst) = dequant_fp8x8(st_k[i].x, st_k[i].y, st_ks[i]);
         *reinterpret_cast<uint4*>(kdst + kTileBytes) = dequant_fp8x8(st_v[i].x, st_v[i].y, st_vs[i]);
       }
@@ -671,7 +671,7 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
   // into the registers the finished exponentials have just released, so the new scores are in
   // place for the next iteration without moves.
   // ------------------------------------------------------------------------------------------
-  constexpr bool PIPELINED = (J == 4) && !KV_FP8;
+  constexpr bool PIPELINED = (J == 4 || J == 8) && !KV_FP8;
   if constexpr (PIPELINED) {
     if (T0 < T1) {
       typedef __attribute__((ext_vector_type(8))) short s16x8;
@@ -688,7 +688,7 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
         char* dst = lds + buf * kBufBytes + wave * 1024;
         __builtin_amdgcn_global_load_lds(
             (const __attribute__((address_space(1))) void*)(kb + ((unsigned long)((unsigned)nslot[i] * kr + lane_ch) << 4)),
-            (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
+            (__attribute__((address_space(3))) void*)(dst + i * (NW * 1024)), 16, 0, 0);
       };
       auto issue_v1 = [&](int t, int buf, int i) __attribute__((always_inline)) {
         const bool ctx = t < Tc;
@@ -697,7 +697,7 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
         char* dst = lds + buf * kBufBytes + kTileBytes + wave * 1024;
         __builtin_amdgcn_global_load_lds(
             (const __attribute__((address_space(1))) void*)(vb + ((unsigned long)((unsigned)nsv[i] * vr + lane_ch) << 4)),
-            (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
+            (__attribute__((address_space(3))) void*)(dst + i * (NW * 1024)), 16, 0, 0);
       };
       auto issue_k = [&](int t, int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -839,9 +839,9 @@ __global__ __launch_bounds__(kThreads, (KV_FP8 || J == 8) ? 1 : 2) void attn_fwd
               exp_pair(stp);
             }
             if (stp + PF < NS) rdk(kf[stp % PF], stp + PF);
-            if ((stp & 1) == 1) {
-              if (stp < 8) issue_v1(t + 1, PAR ^ 1, stp >> 1);
-              else if (k_on) issue_k1(t + 2, PAR, (stp >> 1) - 4);
+            if ((stp & 1) == 1 && ((stp & 7) >> 1) < kDmaGroups) {
+              if (stp < 8) issue_v1(t + 1, PAR ^ 1, (stp & 7) >> 1);
+              else if (k_on) issue_k1(t + 2, PAR, (stp & 7) >> 1);
             }
             __builtin_amdgcn_sched_barrier(0);
           }
@@ -1237,16 +1237,18 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   const long units = (long)d->n_req * d->num_kv_heads;
   const bool fp8 = !prefill && d->k_cache != nullptr && d->max_ctx_len > 0 && d->kv_dtype == PDLLM_KV_FP8_E4M3;
   const int cus = 256;
-  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 1.5;
+  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 1.5, kWide = 1.2;
   constexpr int kStaticLds = 66 * 1024;
   static const int js[] = {1, 2, 4, 5, 6, 8};
-  static const double upw[] = {0.25, 0.5, 1.0, 1.25, 1.5, 2.0};
+  static const double upw[] = {0.25, 0.5, 1.0, 1.25, 1.5, 1.0};
   AttnPlan best = {4, 1, (int)T, (int)T, (int)T, 1, 1};
   double best_cost = 1e300;
   for (int ji = 0; ji < 6; ++ji) {
     const int J = js[ji];
     if (d->rows_per_group && d->rows_per_group != 32 * J) continue;
-    if (!d->rows_per_group && (J == 5 || J == 6 || J == 8)) continue;  // too many registers for two workgroups per CU: only on request
+    if (!d->rows_per_group && (J == 5 || J == 6)) continue;  // too many registers for two workgroups per CU: only on request
+    if (J == 8 && fp8) continue;  // the 8-wave workgroup has no room for the fp8 staging registers
+    if (J == 8 && prefill && !d->rows_per_group) continue;  // coarser causal staircase: measured slower
     const long row_tiles = (nblk + J - 1) / J;
     const long cols = units * row_tiles;
     const bool two = !fp8 && J != 8 && kStaticLds + dyn_lds_bytes(J, d->mask_mode) <= 80 * 1024;
@@ -1284,7 +1286,8 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
       if (n_lin >= (1l << 30)) continue;
       const long grid = (n_lin + span - 1) / span;
       const long n = (grid + cus - 1) / cus;  // workgroups on the most loaded CU
-      const double serial = two ? (double)(n / 2) * 2.0 * kPair + (double)(n % 2) : (double)n;
+      // an 8-wave workgroup behaves like a co-resident pair that shares its tiles
+      const double serial = J == 8 ? (double)n * kWide : two ? (double)(n / 2) * 2.0 * kPair + (double)(n % 2) : (double)n;
       const bool cut = span < t_lin;
       const long pieces = cut ? (t_lin + span - 1) / span + (t_lin % span ? 1 : 0) : 1;
       double cost = serial * ((double)span * (kFixed + upw[ji]) + kPiece * (cut && t_lin % span ? 2.0 : 1.0)) + 1.0;
@@ -1404,7 +1407,7 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
   p.scale_log2 = d->sm_scale * 1.4426950408889634f;
 
   if (plan.grid <= 0) return PDLLM_ERR_SHAPE;
-  const dim3 grid((unsigned)plan.grid), block(kThreads);
+  const dim3 grid((unsigned)plan.grid), block(plan.J == 8 ? 512 : kThreads);
   const bool fp8 = has_cache && d->kv_dtype == PDLLM_KV_FP8_E4M3;
   const int dyn = dyn_lds_bytes(plan.J, d->mask_mode);
 #define PDLLM_LAUNCH(JJ)                                                                              \
