@@ -127,7 +127,7 @@ typedef struct pdllm_attn_desc {
   int32_t kv_dtype;    /* PDLLM_KV_*  (dtype of the cache; in-flight K/V are bf16) */
   int32_t mask_mode;   /* PDLLM_MASK_*                                        */
   int32_t num_splits;  /* 0 = choose; 1..16 = cut every column into this many equal KV splits */
-  int32_t rows_per_group; /* 0 = choose; else 32*J, J in {1,2,4,5,6,8}        */
+  int32_t rows_per_group; /* 0 = choose; else 32*J, J in {1,2,4,5,6,8} rows per workgroup (8: 512 threads) */
   float sm_scale;      /* softmax scale (1/sqrt(d) when the caller has no own) */
   /* optional: the slot table of the visible prefix, built by pdllm_attn_build_slot_table from
    * block_table and the ranges.  It only depends on those, so one table serves every layer of

@@ -249,7 +249,6 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
   constexpr int NW = J == 8 ? 8 : 4;        // wavefronts per workgroup
   constexpr int kDmaGroups = 16 / NW;       // a tile is 16 groups of 4 rows; a wave copies this many of them
   constexpr bool HAS_A = J >= 4;
-  constexpr bool DUAL = false;
   constexpr bool HAS_B = J != 4 && J != 8;
   constexpr int GS = (J == 1 || J == 5) ? 4 : (J == 2 || J == 6) ? 2 : 1;  // waves sharing a B block
   constexpr bool QB_LDS = J == 5 || J == 6;  // Q of the shared block(s) lives in LDS, not in registers
@@ -496,12 +495,10 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
   };
 
   // ---- one pass: row block(s) x NKB key blocks of the tile in LDS ----
-  // dual: slot B uses the same key blocks and rides on the operand fragments slot A reads.
   // Operand reads run two steps ahead of the MFMAs; the scheduling barriers keep that order.
-  auto pass = [&](bool generic, auto nkb_tag, auto dual_tag, auto fora_tag, int kb_first, int bufoff,
+  auto pass = [&](bool generic, auto nkb_tag, auto fora_tag, int kb_first, int bufoff,
                   int nvalid, bool active, int a0, int par) __attribute__((always_inline)) {
     constexpr int NKB = decltype(nkb_tag)::value;
-    constexpr bool DUAL2 = decltype(dual_tag)::value;
     constexpr bool forA = decltype(fora_tag)::value;
     constexpr bool QLDS = QB_LDS && !forA;
     const int kbase_bytes = bufoff + kb_first * 32 * kRowBytes;
@@ -514,14 +511,12 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
 
     // the accumulators start at minus the running maximum
     const float i1 = (M1 == -INFINITY) ? 0.f : -M1;
-    const float i2 = (MB == -INFINITY) ? 0.f : -MB;
-    f32x16 S1[NKB], S2[DUAL2 ? NKB : 1];
+    f32x16 S1[NKB];
 #pragma unroll
     for (int b = 0; b < NKB; ++b)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         S1[b][i] = i1;
-        if constexpr (DUAL2) S2[b][i] = i2;
       }
     if constexpr (!QLDS) {
       constexpr int PF = 4;  // operand reads run PF steps ahead of the MFMAs (LDS latency ~ 3-4 MFMAs)
@@ -547,7 +542,6 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
         else lds_wait<0>(kf[stp % PF]);
         const bf16x8 cur = kf[stp % PF];
         S1[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, Q1[ks], S1[kb], 0, 0, 0);
-        if constexpr (DUAL2) S2[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, QB[ks], S2[kb], 0, 0, 0);
         if (stp + PF < NS) rdk(kf[stp % PF], stp + PF);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -574,7 +568,7 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
       }
     }
 
-    bf16x8 P1[NKB][2], P2[DUAL2 ? NKB : 1][2];
+    bf16x8 P1[NKB][2];
     const bool causal_here = active && p.mask_mode == PDLLM_MASK_CAUSAL;
     const bool dense_here = active && p.mask_mode == PDLLM_MASK_DENSE;
     {
@@ -583,14 +577,6 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
       int tl = srow1 - tq_first;
       tl = tl < 0 ? 0 : (tl >= kMaxTok ? kMaxTok - 1 : tl);
       softmax_update<NKB>(S1, P1, O1, M1, l1, h, kb_first, generic, lim,
-                          dense_here ? &s_maskbits[par][tl][0] : nullptr);
-    }
-    if constexpr (DUAL2) {
-      int lim = nvalid;
-      if (causal_here) { const int cl = srowB - a0 + 1; lim = cl < lim ? cl : lim; }
-      int tl = srowB - tq_first;
-      tl = tl < 0 ? 0 : (tl >= kMaxTok ? kMaxTok - 1 : tl);
-      softmax_update<NKB>(S2, P2, OB, MB, lB, h, kb_first, generic, lim,
                           dense_here ? &s_maskbits[par][tl][0] : nullptr);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -623,7 +609,6 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
         const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
         const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
         O1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P1[kj >> 1][kj & 1], O1[db], 0, 0, 0);
-        if constexpr (DUAL2) OB[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P2[kj >> 1][kj & 1], OB[db], 0, 0, 0);
         if (stp + 2 < NS) { rdv(lo[stp & 1], stp + 2, 0); rdv(hi[stp & 1], stp + 2, 1); }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -638,14 +623,12 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
     nvalid = nvalid < kKT ? nvalid : kKT;
     using N1 = std::integral_constant<int, 1>;
     using NT = std::integral_constant<int, kNKB>;
-    using Dual = std::integral_constant<bool, DUAL>;
-    using Single = std::integral_constant<bool, false>;
     if (has_next) issue_tile(t + 1, buf ^ 1);
     if (t + 2 < T1) load_slots(t + 2);
-    if (HAS_A) pass(generic, NT{}, Dual{}, std::true_type{}, 0, bufoff, nvalid, active, a0, buf);
-    if (HAS_B && !DUAL) {
+    if (HAS_A) pass(generic, NT{}, std::true_type{}, 0, bufoff, nvalid, active, a0, buf);
+    if (HAS_B) {
       if (GS == 2 || ((t & 1) == parB))
-        pass(generic, N1{}, Single{}, std::false_type{}, kbB, bufoff, nvalid, active, a0, buf);
+        pass(generic, N1{}, std::false_type{}, kbB, bufoff, nvalid, active, a0, buf);
     }
   };
 
@@ -1246,7 +1229,8 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   for (int ji = 0; ji < 6; ++ji) {
     const int J = js[ji];
     if (d->rows_per_group && d->rows_per_group != 32 * J) continue;
-    if (!d->rows_per_group && (J == 5 || J == 6)) continue;  // too many registers for two workgroups per CU: only on request
+    // 5 and 6 row blocks need more than 256 registers: fine for the fp8 path (one workgroup per CU anyway), else only on request
+    if (!d->rows_per_group && (J == 5 || J == 6) && !fp8) continue;
     if (J == 8 && fp8) continue;  // the 8-wave workgroup has no room for the fp8 staging registers
     if (J == 8 && prefill && !d->rows_per_group) continue;  // coarser causal staircase: measured slower
     const long row_tiles = (nblk + J - 1) / J;
