@@ -313,7 +313,8 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
   const int wg_last = ((col + 1) * p.t_lin - 1) / p.span;
   const int piece = wg - wg_first;
   const bool whole = wg_first == wg_last;  // the only piece: write the result, not a partial
-  const int row_tile = col % p.row_tiles;
+  // causal: the row groups that see the most keys are dispatched first, the short ones fill the tail
+  const int row_tile = p.mask_mode == PDLLM_MASK_CAUSAL ? p.row_tiles - 1 - col % p.row_tiles : col % p.row_tiles;
   const int kvh = (col / p.row_tiles) % p.Hkv;
   const int req = col / (p.row_tiles * p.Hkv);
 
@@ -735,17 +736,20 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
           int tl = srowA - tq_first;
           tl = tl < 0 ? 0 : (tl >= kMaxTok ? kMaxTok - 1 : tl);
           const uint32_t* mrow = (active && p.mask_mode == PDLLM_MASK_DENSE) ? &s_maskbits[PAR][tl][0] : nullptr;
+          // a causal tile that lies below the diagonal for every row of this wave needs no mask
+          if (mrow != nullptr || __builtin_amdgcn_ballot_w64(lim < kKT) != 0) {
 #pragma unroll
-          for (int b = 0; b < 2; ++b) {
-            const int lb = lim - 32 * b;
-            uint32_t W = lb >= 32 ? 0xffffffffu : (lb <= 0 ? 0u : ((1u << lb) - 1u));
-            if (mrow != nullptr) W &= mrow[b];
-            W >>= 4 * h;
+            for (int b = 0; b < 2; ++b) {
+              const int lb = lim - 32 * b;
+              uint32_t W = lb >= 32 ? 0xffffffffu : (lb <= 0 ? 0u : ((1u << lb) - 1u));
+              if (mrow != nullptr) W &= mrow[b];
+              W >>= 4 * h;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              constexpr uint32_t one = 1u;
-              const uint32_t bit = one << (8 * (i >> 2) + (i & 3));
-              Sc[b][i] = (W & bit) ? Sc[b][i] : -INFINITY;
+              for (int i = 0; i < 16; ++i) {
+                constexpr uint32_t one = 1u;
+                const uint32_t bit = one << (8 * (i >> 2) + (i & 3));
+                Sc[b][i] = (W & bit) ? Sc[b][i] : -INFINITY;
+              }
             }
           }
         }
@@ -1067,7 +1071,7 @@ struct MergeParams {
   __bf16* out;
   const int* q_start_loc;
   long o_stride, n_tokens;
-  int n_req, max_q_len, Hq, Hkv, rows_per_group, row_tiles, t_lin, span, max_pieces;
+  int n_req, max_q_len, Hq, Hkv, rows_per_group, row_tiles, t_lin, span, max_pieces, reversed;
 };
 
 __global__ __launch_bounds__(256) void attn_merge_kernel(const MergeParams m) {
@@ -1085,7 +1089,8 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const MergeParams m) {
   if (q0 < 0 || tq >= Sq || (long)q0 + Sq > m.n_tokens || Sq > m.max_q_len) return;
   const int G = m.Hq / m.Hkv;
   const int kvh = head / G;
-  const int col = (req * m.Hkv + kvh) * m.row_tiles + (tq * G + (head - kvh * G)) / m.rows_per_group;
+  const int rt = (tq * G + (head - kvh * G)) / m.rows_per_group;
+  const int col = (req * m.Hkv + kvh) * m.row_tiles + (m.reversed ? m.row_tiles - 1 - rt : rt);
   const int first = (col * m.t_lin) / m.span;
   const int np = ((col + 1) * m.t_lin - 1) / m.span - first + 1;
   if (np == 1) return;
@@ -1416,7 +1421,7 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
     m.ws_o = p.ws_o; m.ws_lse = p.ws_lse; m.out = p.out; m.q_start_loc = p.q_start_loc;
     m.o_stride = p.o_stride; m.n_tokens = p.n_tokens;
     m.n_req = p.n_req; m.max_q_len = p.max_q_len; m.Hq = p.Hq; m.Hkv = p.Hkv;
-    m.rows_per_group = 32 * plan.J; m.row_tiles = plan.row_tiles;
+    m.rows_per_group = 32 * plan.J; m.row_tiles = plan.row_tiles; m.reversed = p.mask_mode == PDLLM_MASK_CAUSAL;
     m.t_lin = plan.t_lin; m.span = plan.span; m.max_pieces = plan.max_pieces;
     const long mrows = (long)d->n_req * d->max_q_len * d->num_q_heads;
     hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((mrows + 7) / 8)), dim3(256), 0, stream, m);
