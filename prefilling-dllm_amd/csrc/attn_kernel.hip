@@ -100,8 +100,15 @@ struct AttnKParams {
   // n_cols * t_lin positions that is cut into spans of `span` tiles, one per workgroup
   int t_lin;       // positions per column (>= the largest tile count of a column)
   int span;        // tiles per workgroup
-  int n_lin;       // n_cols * t_lin
+  int n_lin;       // length of the line
   int max_pieces;  // partial results per row in the workspace
+  // head == 0: one line over all columns (n_lin = columns * t_lin).  head > 0: the row_tiles columns of
+  // one (request, KV head), which read the same K/V tiles, form a set of wg_set workgroups: the first
+  // row_tiles of them take the first `head` tiles of one column each, side by side over the same
+  // tiles, which they share in L2; the others cut the line of the columns' remaining t_lin - head
+  // tiles (n_lin = row_tiles * (t_lin - head) positions) into spans.
+  int head;
+  int wg_set;
   int max_q_len;
   float scale_log2;  // sm_scale * log2(e)
 };
@@ -302,17 +309,40 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
   // this workgroup's span of the tile line; it may cover the end of one column and the start of
   // the next, each part ("piece") is an attention pass of its own
   const int wg = xcd_remap(blockIdx.x, gridDim.x);
-  int x = wg * p.span;
-  const int x_end = x + p.span < p.n_lin ? x + p.span : p.n_lin;
-  while (x < x_end) {
-  const int col = x / p.t_lin;
-  const int tb = x - col * p.t_lin;
-  const int te = tb + (x_end - x) < p.t_lin ? tb + (x_end - x) : p.t_lin;
-  x += te - tb;
-  const int wg_first = (col * p.t_lin) / p.span;            // workgroups holding pieces of this column
-  const int wg_last = ((col + 1) * p.t_lin - 1) / p.span;
-  const int piece = wg - wg_first;
-  const bool whole = wg_first == wg_last;  // the only piece: write the result, not a partial
+  int col0 = 0;      // first column of the line this workgroup works on
+  int head_rt = -1;  // >= 0: this workgroup takes the head of that column of its set and nothing else
+  int y;
+  if (p.head > 0) {
+    const int set = wg / p.wg_set;
+    const int j = wg - set * p.wg_set;
+    col0 = set * p.row_tiles;
+    head_rt = j < p.row_tiles ? j : -1;
+    y = j < p.row_tiles ? p.n_lin : (j - p.row_tiles) * p.span;
+  } else {
+    y = wg * p.span;
+  }
+  const int y_end = y + p.span < p.n_lin ? y + p.span : p.n_lin;
+  const int tail_len = p.t_lin - p.head;  // positions of a column after its head
+  while (head_rt >= 0 || y < y_end) {
+  int rt_lin, tb, te;
+  if (head_rt >= 0) {
+    rt_lin = head_rt;
+    tb = 0;
+    te = p.head;
+    head_rt = -1;
+  } else {
+    rt_lin = y / tail_len;
+    tb = p.head + (y - rt_lin * tail_len);
+    // (the divisions run on the vector unit: bring the results back to scalar registers)
+    tb = __builtin_amdgcn_readfirstlane(tb);
+    te = tb + (y_end - y) < p.t_lin ? tb + (y_end - y) : p.t_lin;
+    y += te - tb;
+  }
+  const int col = __builtin_amdgcn_readfirstlane(col0 + rt_lin);
+  // The head of a column is its piece 0.  A later piece starts at a workgroup boundary, so its
+  // number is the count of boundaries since the start of the column's tail.
+  const int piece = __builtin_amdgcn_readfirstlane(tb < p.head ? 0 : (p.head > 0 ? 1 : 0) + (tb - p.head + p.span - 1) / p.span);
+  const bool whole = tb == 0 && te == p.t_lin;  // the only piece: write the result, not a partial
   // causal: the row groups that see the most keys are dispatched first, the short ones fill the tail
   const int row_tile = p.mask_mode == PDLLM_MASK_CAUSAL ? p.row_tiles - 1 - col % p.row_tiles : col % p.row_tiles;
   const int kvh = (col / p.row_tiles) % p.Hkv;
@@ -1071,7 +1101,7 @@ struct MergeParams {
   __bf16* out;
   const int* q_start_loc;
   long o_stride, n_tokens;
-  int n_req, max_q_len, Hq, Hkv, rows_per_group, row_tiles, t_lin, span, max_pieces, reversed;
+  int n_req, max_q_len, Hq, Hkv, rows_per_group, row_tiles, t_lin, span, max_pieces, reversed, head;
 };
 
 __global__ __launch_bounds__(256) void attn_merge_kernel(const MergeParams m) {
@@ -1091,8 +1121,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const MergeParams m) {
   const int kvh = head / G;
   const int rt = (tq * G + (head - kvh * G)) / m.rows_per_group;
   const int col = (req * m.Hkv + kvh) * m.row_tiles + (m.reversed ? m.row_tiles - 1 - rt : rt);
-  const int first = (col * m.t_lin) / m.span;
-  const int np = ((col + 1) * m.t_lin - 1) / m.span - first + 1;
+  const int tail_len = m.t_lin - m.head;
+  const int tail_at = (m.head > 0 ? col % m.row_tiles : col) * tail_len;  // on the line the column's tail lies on
+  const int np = (m.head > 0 ? 1 : 0) + (tail_at + tail_len - 1) / m.span - tail_at / m.span + 1;
   if (np == 1) return;
   const long R = ((long)(q0 + tq) * m.Hq + head) * m.max_pieces;
   float M = -INFINITY;
@@ -1137,6 +1168,8 @@ struct AttnPlan {
   int n_lin;       // columns * t_lin
   int max_pieces;  // most pieces a column is cut into
   int grid;        // workgroups
+  int head;        // tiles of a column taken by a workgroup of its own at the start of its set (0: one line over all columns)
+  int wg_set;      // workgroups per set when head > 0
 };
 
 static int ilog2_exact(int v) {
@@ -1229,7 +1262,7 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   constexpr int kStaticLds = 66 * 1024;
   static const int js[] = {1, 2, 4, 5, 6, 8};
   static const double upw[] = {0.25, 0.5, 1.0, 1.25, 1.5, 1.0};
-  AttnPlan best = {4, 1, (int)T, (int)T, (int)T, 1, 1};
+  AttnPlan best = {4, 1, (int)T, (int)T, (int)T, 1, 1, 0, 0};
   double best_cost = 1e300;
   for (int ji = 0; ji < 6; ++ji) {
     const int J = js[ji];
@@ -1243,8 +1276,8 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
     const bool two = !fp8 && J != 8 && kStaticLds + dyn_lds_bytes(J, d->mask_mode) <= 80 * 1024;
     const long slots = (long)cus * (two ? 2 : 1);
     // candidate spans: whole columns, columns cut into 2..16 equal parts, and the balanced cut
-    for (int cand = 0; cand <= 18; ++cand) {
-      long t_lin = T, span;
+    for (int cand = 0; cand <= 20; ++cand) {
+      long t_lin = T, span, head = 0, wg_set = 0;
       if (cand == 0) {
         span = T;
       } else if (cand <= 15) {
@@ -1260,9 +1293,21 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
         if (prefill) continue;
         span = (cols * T + 2 * slots - 1) / (2 * slots);
         if (span >= T || span < 4) continue;
-      } else {
+      } else if (cand == 18) {
         if (d->tiles_per_workgroup <= 0) continue;
         span = d->tiles_per_workgroup < T ? d->tiles_per_workgroup : T;
+      } else {
+        // the balanced cut, set by set: k workgroups per (request, KV head), the first row_tiles of
+        // them side by side over the same leading tiles of their columns
+        if (prefill || row_tiles < 2) continue;
+        const long k = (cand == 19 ? slots : 2 * slots) / units;
+        if (k <= row_tiles) continue;
+        // a head workgroup handles one piece, the others two or three: it takes kHeadExtra tiles more
+        constexpr long kHeadExtra = 3;
+        span = (row_tiles * (T - kHeadExtra) + k - 1) / k;
+        head = span + kHeadExtra;
+        if (head >= T || span < 4) continue;
+        wg_set = k;
       }
       if (d->tiles_per_workgroup > 0) {
         if (cand != 18) continue;
@@ -1271,14 +1316,22 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
       } else if (prefill && cand != 0) {
         continue;
       }
-      const long n_lin = cols * t_lin;
+      const long n_lin = head > 0 ? row_tiles * (t_lin - head) : cols * t_lin;
       if (n_lin >= (1l << 30)) continue;
-      const long grid = (n_lin + span - 1) / span;
+      const long grid = head > 0 ? units * wg_set : (n_lin + span - 1) / span;
       const long n = (grid + cus - 1) / cus;  // workgroups on the most loaded CU
       // an 8-wave workgroup behaves like a co-resident pair that shares its tiles
       const double serial = J == 8 ? (double)n * kWide : two ? (double)(n / 2) * 2.0 * kPair + (double)(n % 2) : (double)n;
       const bool cut = span < t_lin;
-      const long pieces = cut ? (t_lin + span - 1) / span + (t_lin % span ? 1 : 0) : 1;
+      long pieces = cut ? (t_lin + span - 1) / span + (t_lin % span ? 1 : 0) : 1;
+      if (head > 0) {
+        pieces = 0;
+        for (long r = 0; r < row_tiles; ++r) {
+          const long a = r * (t_lin - head);
+          const long np = 1 + (a + t_lin - head - 1) / span - a / span + 1;
+          pieces = np > pieces ? np : pieces;
+        }
+      }
       double cost = serial * ((double)span * (kFixed + upw[ji]) + kPiece * (cut && t_lin % span ? 2.0 : 1.0)) + 1.0;
       if (cut) {
         // fp32 partials written and read back (~4 MB per unit of time), plus the merge launch
@@ -1286,6 +1339,7 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
         const double part_bytes = (double)units * rows * avg_pieces * (kD + 1) * 4.0 * 2.0;
         cost += part_bytes / 4.0e6 + 4.0;
       }
+      if (head > 0) cost *= 0.97;  // the set's workgroups share their tiles in L2: less traffic for the same cut
       if (cost < best_cost) {
         best_cost = cost;
         best.J = J;
@@ -1295,13 +1349,15 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
         best.n_lin = (int)n_lin;
         best.max_pieces = (int)pieces;
         best.grid = (int)grid;
+        best.head = (int)head;
+        best.wg_set = (int)wg_set;
       }
     }
   }
   if (best_cost == 1e300) {
     // the forced values fit no candidate (e.g. a split of a prefill): one workgroup per column, J = 4
     const long row_tiles = (nblk + 3) / 4;
-    best = {4, (int)row_tiles, (int)T, (int)T, (int)(units * row_tiles * T), 1, (int)(units * row_tiles)};
+    best = {4, (int)row_tiles, (int)T, (int)T, (int)(units * row_tiles * T), 1, (int)(units * row_tiles), 0, 0};
   }
   return best;
 }
@@ -1392,6 +1448,8 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
   p.span = plan.span;
   p.n_lin = plan.n_lin;
   p.max_pieces = plan.max_pieces;
+  p.head = plan.head;
+  p.wg_set = plan.wg_set;
   p.max_q_len = d->max_q_len;
   p.scale_log2 = d->sm_scale * 1.4426950408889634f;
 
@@ -1422,7 +1480,7 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
     m.o_stride = p.o_stride; m.n_tokens = p.n_tokens;
     m.n_req = p.n_req; m.max_q_len = p.max_q_len; m.Hq = p.Hq; m.Hkv = p.Hkv;
     m.rows_per_group = 32 * plan.J; m.row_tiles = plan.row_tiles; m.reversed = p.mask_mode == PDLLM_MASK_CAUSAL;
-    m.t_lin = plan.t_lin; m.span = plan.span; m.max_pieces = plan.max_pieces;
+    m.t_lin = plan.t_lin; m.span = plan.span; m.max_pieces = plan.max_pieces; m.head = plan.head;
     const long mrows = (long)d->n_req * d->max_q_len * d->num_q_heads;
     hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((mrows + 7) / 8)), dim3(256), 0, stream, m);
     st = launch_status();
