@@ -186,7 +186,7 @@ def secondary_shapes(torch, ops, dev):
     V2 = 152064
     logits = (torch.randn((32, 4, V2), generator=gd, device=dev) * 2.0).to(torch.bfloat16)
     labels = torch.randint(0, V2, (32, 4), generator=gd, device=dev)
-    us = _time_us(torch, lambda: ops.topk_lowest_index(ops.chunk_scores_from_logits(logits, labels), 4))
+    us = _time_us(torch, lambda: ops.chunk_select_from_logits(logits, labels, 4))
     by = logits.numel() * 2
     out["score_32x4x152064_top4"] = {"us": us, "hbm_GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS}
     probs = torch.softmax(torch.randn((8, HQ, 64, 1025), generator=gd, device=dev), dim=-1)
@@ -201,9 +201,8 @@ def secondary_shapes(torch, ops, dev):
     ids = torch.full((4, 32), V5 - 1, dtype=torch.int64, device=dev)
 
     def unmask():
-        conf, tok = ops.conf_argmax(lg, 32)
         ids.fill_(V5 - 1)
-        ops.threshold_unmask(conf, tok, ids, V5 - 1, 0.9)
+        ops.denoise_unmask(lg, ids, V5 - 1, 0.9)
     us = _time_us(torch, unmask)
     by = lg.numel() * 2
     out["unmask_4x32x126464"] = {"us": us, "hbm_GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS}

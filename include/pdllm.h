@@ -200,6 +200,17 @@ int64_t pdllm_vocab_workspace_bytes(int64_t n_rows, int64_t vocab);
 int pdllm_chunk_score_reduce(const float* logp, int64_t n_chunks, int64_t rows_per_chunk,
                              int32_t mean, float* scores_out, pdllm_stream_t stream);
 
+/* score_chunk_self_information_engine + the ranking of select_chunks_by_engine in one call
+ * (ENG:1148-1152 and 1199-1204; the reference runs them back to back for every draft round):
+ * pdllm_selfinfo_logprob over [n_chunks * rows_per_chunk, vocab] logits, pdllm_chunk_score_reduce
+ * and pdllm_topk_lowest_index of the n_chunks scores, as two launches; same results as the three
+ * calls.  logp_out may be NULL.  n_chunks <= 1024, 1 <= k <= n_chunks; workspace as
+ * pdllm_vocab_workspace_bytes(n_chunks * rows_per_chunk, vocab). */
+int pdllm_chunk_select(const void* logits, int64_t logits_stride, const int64_t* labels,
+                       int64_t n_chunks, int64_t rows_per_chunk, int64_t vocab, int32_t mean, int64_t k,
+                       int32_t sorted_ascending, void* workspace, int64_t workspace_bytes,
+                       float* logp_out, float* scores_out, int64_t* indices_out, pdllm_stream_t stream);
+
 /* Replaces the ranking of select_chunks_by_engine (ENG:1199-1204): per row of
  * scores [n_rows, n] (non-finite -> -inf), the k best indices by (score desc,
  * index asc), returned ascending when sorted_ascending != 0, else in rank order.
@@ -294,6 +305,15 @@ int pdllm_threshold_unmask(const float* conf, const int64_t* token, int64_t* blo
                            int64_t n_seqs, int64_t block_len, int64_t mask_token_id,
                            float threshold, uint8_t* transfer_out, int32_t* n_masked_left,
                            pdllm_stream_t stream);
+
+/* One denoise step's sampling and transfer (ENG:1647-1681 followed by 2146-2157) in one call:
+ * pdllm_conf_argmax and pdllm_threshold_unmask as two launches, same results; conf_out and
+ * token_out [n_seqs * block_len] are written as by pdllm_conf_argmax. */
+int pdllm_denoise_unmask(const void* logits, int64_t logits_stride, const void* last_logit,
+                         int64_t last_logit_stride, int64_t n_seqs, int64_t block_len, int64_t vocab,
+                         int32_t shift, int64_t* block_ids, int64_t mask_token_id, float threshold,
+                         void* workspace, int64_t workspace_bytes, float* conf_out, int64_t* token_out,
+                         uint8_t* transfer_out, int32_t* n_masked_left, pdllm_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * Rotary embedding (the step in front of the path)                           *

@@ -76,13 +76,14 @@ __global__ __launch_bounds__(256) void vocab_partial_kernel(
           x[2 * k] = bf16_bits_to_f32(w[k] & 0xffffu);
           x[2 * k + 1] = bf16_bits_to_f32(w[k] >> 16);
         }
-        // vector step: one rescale for the 8 values
-        float vm = x[0];
-        int vi = 0;
-#pragma unroll
-        for (int k = 1; k < 8; ++k)
-          if (x[k] > vm) { vm = x[k]; vi = k; }
+        // vector step: one rescale for the 8 values; the position of a new maximum is only looked
+        // for when there is one (rare once the running maximum has settled)
+        const float vm = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
         if (vm > st.m) {
+          int vi = 7;
+#pragma unroll
+          for (int k = 6; k >= 0; --k)
+            if (x[k] == vm) vi = k;  // first position of the maximum
           st.s *= __builtin_amdgcn_exp2f((st.m - vm) * kLog2e);
           st.m = vm;
           st.idx = i + vi;
@@ -129,6 +130,27 @@ __global__ __launch_bounds__(256) void vocab_partial_kernel(
   }
 }
 
+// the split partials of a row, combined in split order
+__device__ __forceinline__ RowStat row_stat(const float* __restrict__ part_m, const float* __restrict__ part_s,
+                                            const long* __restrict__ part_idx, int nsplit, long row) {
+  RowStat a = {part_m[row * nsplit], part_s[row * nsplit], part_idx[row * nsplit]};
+  for (int s = 1; s < nsplit; ++s) {
+    RowStat b = {part_m[row * nsplit + s], part_s[row * nsplit + s], part_idx[row * nsplit + s]};
+    stat_merge(a, b);
+  }
+  return a;
+}
+
+// log-softmax of the label: logits[row, label] - logsumexp(row); labels outside the vocabulary give -inf
+__device__ __forceinline__ float label_logprob(const RowStat& a, const __bf16* __restrict__ logits,
+                                               long logits_stride, const long* __restrict__ labels, long vocab,
+                                               long row) {
+  const long lab = labels[row];
+  if (lab < 0 || lab >= vocab) return -INFINITY;
+  const float x = bf16_bits_to_f32(__builtin_bit_cast(unsigned short, logits[row * logits_stride + lab]));
+  return (x - a.m) - __log2f(a.s) * kLn2;
+}
+
 // mode 0: logp[row] = logits[row, label] - logsumexp ; mode 1: conf = 1 / sum exp(x - max), token = argmax
 __global__ __launch_bounds__(64) void vocab_final_kernel(
     const float* __restrict__ part_m, const float* __restrict__ part_s, const long* __restrict__ part_idx,
@@ -136,19 +158,9 @@ __global__ __launch_bounds__(64) void vocab_final_kernel(
     const long* __restrict__ labels, long vocab, float* __restrict__ out_f, long* __restrict__ out_i) {
   const long row = (long)blockIdx.x * 64 + threadIdx.x;
   if (row >= n_rows) return;
-  RowStat a = {part_m[row * nsplit], part_s[row * nsplit], part_idx[row * nsplit]};
-  for (int s = 1; s < nsplit; ++s) {
-    RowStat b = {part_m[row * nsplit + s], part_s[row * nsplit + s], part_idx[row * nsplit + s]};
-    stat_merge(a, b);
-  }
+  const RowStat a = row_stat(part_m, part_s, part_idx, nsplit, row);
   if (mode == 0) {
-    const long lab = labels[row];
-    float r = -INFINITY;
-    if (lab >= 0 && lab < vocab) {
-      const float x = bf16_bits_to_f32(__builtin_bit_cast(unsigned short, logits[row * logits_stride + lab]));
-      r = (x - a.m) - __log2f(a.s) * kLn2;
-    }
-    out_f[row] = r;
+    out_f[row] = label_logprob(a, logits, logits_stride, labels, vocab, row);
   } else {
     out_f[row] = 1.f / a.s;
     out_i[row] = a.idx;
@@ -163,6 +175,119 @@ __global__ __launch_bounds__(64) void chunk_score_reduce_kernel(const float* __r
   float acc = 0.f;
   for (long j = 0; j < rows_per_chunk; ++j) acc += logp[c * rows_per_chunk + j];
   out[c] = mean ? acc / (float)rows_per_chunk : acc;
+}
+
+// Tail of the chunk scoring in one workgroup: row log-probabilities from the split partials, chunk
+// scores (rows added in index order, optionally the mean), and the k best chunks by (score
+// descending, index ascending; non-finite scores count as -inf), written in ascending index order
+// or best first.  n_chunks <= kSelectMax.
+constexpr int kSelectMax = 1024;
+constexpr int kSelectRows = 4096;
+__global__ __launch_bounds__(256) void score_select_kernel(
+    const float* __restrict__ part_m, const float* __restrict__ part_s, const long* __restrict__ part_idx,
+    int nsplit, long n_chunks, long rows_per_chunk, int mean, const __bf16* __restrict__ logits,
+    long logits_stride, const long* __restrict__ labels, long vocab, long k, int sorted_ascending,
+    float* __restrict__ logp_out, float* __restrict__ scores_out, long* __restrict__ idx_out) {
+  __shared__ uint64_t keys[kSelectMax];
+  __shared__ uint8_t taken[kSelectMax];
+  __shared__ float row_lp[kSelectRows];
+  const long n_rows = n_chunks * rows_per_chunk;
+  const bool staged = n_rows <= kSelectRows;  // one thread per row first, so that the loads of the rows overlap
+  if (staged) {
+    for (long row = threadIdx.x; row < n_rows; row += 256) {
+      const RowStat a = row_stat(part_m, part_s, part_idx, nsplit, row);
+      const float r = label_logprob(a, logits, logits_stride, labels, vocab, row);
+      if (logp_out) logp_out[row] = r;
+      row_lp[row] = r;
+    }
+    __syncthreads();
+  }
+  for (long c = threadIdx.x; c < n_chunks; c += 256) {
+    float acc = 0.f;
+    for (long j = 0; j < rows_per_chunk; ++j) {
+      const long row = c * rows_per_chunk + j;
+      float r;
+      if (staged) {
+        r = row_lp[row];
+      } else {
+        const RowStat a = row_stat(part_m, part_s, part_idx, nsplit, row);
+        r = label_logprob(a, logits, logits_stride, labels, vocab, row);
+        if (logp_out) logp_out[row] = r;
+      }
+      acc += r;
+    }
+    const float score = mean ? acc / (float)rows_per_chunk : acc;
+    scores_out[c] = score;
+    float v = score;
+    if (!(fabsf(v) <= 3.402823466e38f)) v = -INFINITY;
+    // smaller key = better: inverted order-preserving image of the score, then the index
+    uint32_t u = __float_as_uint(v);
+    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    keys[c] = ((uint64_t)(~u) << 32) | (uint32_t)c;
+  }
+  __syncthreads();
+  for (long c = threadIdx.x; c < n_chunks; c += 256) {
+    const uint64_t mine = keys[c];
+    long rank = 0;
+    for (long o = 0; o < n_chunks; ++o) rank += keys[o] < mine ? 1 : 0;
+    taken[c] = rank < k ? 1 : 0;
+    if (!sorted_ascending && rank < k) idx_out[rank] = c;
+  }
+  if (!sorted_ascending) return;
+  __syncthreads();
+  for (long c = threadIdx.x; c < n_chunks; c += 256) {
+    if (!taken[c]) continue;
+    long pos = 0;
+    for (long o = 0; o < c; ++o) pos += taken[o];
+    idx_out[pos] = c;
+  }
+}
+
+// Tail of a denoise step, one wave per block of the batch: confidence (max softmax probability) and
+// argmax token of every position from the split partials, then the transfer rule over the positions
+// that still hold the mask token: the most confident one (lowest index on ties) always, the others
+// when their confidence reaches the threshold.  Writes the tokens into block_ids.
+__global__ __launch_bounds__(64) void unmask_tail_kernel(
+    const float* __restrict__ part_m, const float* __restrict__ part_s, const long* __restrict__ part_idx,
+    int nsplit, long* __restrict__ block_ids, long block_len, long mask_token_id, float threshold,
+    float* __restrict__ conf_out, long* __restrict__ token_out, uint8_t* __restrict__ transfer,
+    int* __restrict__ n_left) {
+  const long b = blockIdx.x;
+  const int lane = threadIdx.x;
+  const long base = b * block_len;
+  float best = -INFINITY;
+  long besti = 0x7fffffffffffffffL;
+  int n_masked = 0;
+  for (long i = lane; i < block_len; i += 64) {
+    const RowStat a = row_stat(part_m, part_s, part_idx, nsplit, base + i);
+    const float c = 1.f / a.s;
+    conf_out[base + i] = c;
+    token_out[base + i] = a.idx;
+    if (block_ids[base + i] == mask_token_id) {
+      ++n_masked;
+      if (c > best || besti == 0x7fffffffffffffffL) { best = c; besti = i; }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const long oi = __shfl_xor(besti, o, 64);
+    n_masked += __shfl_xor(n_masked, o, 64);
+    const bool o_valid = oi != 0x7fffffffffffffffL, s_valid = besti != 0x7fffffffffffffffL;
+    const bool take = o_valid && (!s_valid || ob > best || (ob == best && oi < besti));
+    if (take) { best = ob; besti = oi; }
+  }
+  int moved = 0;
+  for (long i = lane; i < block_len; i += 64) {
+    // this lane wrote conf_out / token_out of position i itself
+    const bool masked = block_ids[base + i] == mask_token_id;
+    const bool t = masked && (i == besti || conf_out[base + i] >= threshold);
+    transfer[base + i] = t ? 1 : 0;
+    if (t) { block_ids[base + i] = token_out[base + i]; ++moved; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) moved += __shfl_xor(moved, o, 64);
+  if (lane == 0 && n_left) n_left[b] = n_masked - moved;
 }
 
 // one wave per block of the batch
@@ -249,7 +374,7 @@ static int vocab_launch(const void* logits, int64_t logits_stride, const void* l
                         int64_t last_stride, int64_t n_rows, int64_t block_len, int64_t vocab, int shift,
                         int mode, const int64_t* labels, void* workspace, int64_t workspace_bytes,
                         float* out_f, int64_t* out_i, hipStream_t stream) {
-  if (!logits || !out_f || !workspace) return PDLLM_ERR_NULL;
+  if (!logits || (!out_f && mode != 2) || !workspace) return PDLLM_ERR_NULL;
   if (mode == 0 && !labels) return PDLLM_ERR_NULL;
   if (mode == 1 && !out_i) return PDLLM_ERR_NULL;
   if (n_rows < 0 || vocab <= 0 || logits_stride < vocab || block_len <= 0) return PDLLM_ERR_SHAPE;
@@ -266,6 +391,7 @@ static int vocab_launch(const void* logits, int64_t logits_stride, const void* l
                      (long)vocab, ns, pm, ps, pi);
   int st = launch_status();
   if (st != PDLLM_OK) return st;
+  if (mode == 2) return PDLLM_OK;  // the caller launches its own tail over the partials
   hipLaunchKernelGGL(vocab_final_kernel, dim3((unsigned)((n_rows + 63) / 64)), dim3(64), 0, stream, pm, ps,
                      pi, ns, (long)n_rows, mode, static_cast<const __bf16*>(logits), (long)logits_stride,
                      reinterpret_cast<const long*>(labels), (long)vocab, out_f,
@@ -339,5 +465,54 @@ extern "C" int pdllm_rope_inplace(void* x, int64_t x_stride, const int64_t* posi
                      static_cast<hipStream_t>(stream), static_cast<__bf16*>(x), (long)x_stride,
                      reinterpret_cast<const long*>(positions), cos_sin_cache, (long)max_positions,
                      (long)n_tokens, n_heads, head_dim);
+  return launch_status();
+}
+
+extern "C" int pdllm_chunk_select(const void* logits, int64_t logits_stride, const int64_t* labels,
+                                  int64_t n_chunks, int64_t rows_per_chunk, int64_t vocab, int32_t mean,
+                                  int64_t k, int32_t sorted_ascending, void* workspace,
+                                  int64_t workspace_bytes, float* logp_out, float* scores_out,
+                                  int64_t* indices_out, pdllm_stream_t stream) {
+  if (!labels || !scores_out || !indices_out) return PDLLM_ERR_NULL;
+  if (n_chunks <= 0 || rows_per_chunk <= 0 || k <= 0 || k > n_chunks) return PDLLM_ERR_SHAPE;
+  if (n_chunks > kSelectMax) return PDLLM_ERR_UNSUPPORTED;
+  const int64_t n_rows = n_chunks * rows_per_chunk;
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  const int st = vocab_launch(logits, logits_stride, nullptr, 0, n_rows, 1, vocab, 0, 2, labels, workspace,
+                              workspace_bytes, nullptr, nullptr, hs);
+  if (st != PDLLM_OK) return st;
+  const int ns = vocab_nsplit(n_rows, vocab);
+  long* pi = static_cast<long*>(workspace);
+  float* pm = reinterpret_cast<float*>(pi + n_rows * ns);
+  float* ps = pm + n_rows * ns;
+  hipLaunchKernelGGL(score_select_kernel, dim3(1), dim3(256), 0, hs, pm, ps, pi, ns, (long)n_chunks,
+                     (long)rows_per_chunk, mean, static_cast<const __bf16*>(logits), (long)logits_stride,
+                     reinterpret_cast<const long*>(labels), (long)vocab, (long)k, sorted_ascending, logp_out,
+                     scores_out, reinterpret_cast<long*>(indices_out));
+  return launch_status();
+}
+
+extern "C" int pdllm_denoise_unmask(const void* logits, int64_t logits_stride, const void* last_logit,
+                                    int64_t last_logit_stride, int64_t n_seqs, int64_t block_len,
+                                    int64_t vocab, int32_t shift, int64_t* block_ids, int64_t mask_token_id,
+                                    float threshold, void* workspace, int64_t workspace_bytes,
+                                    float* conf_out, int64_t* token_out, uint8_t* transfer_out,
+                                    int32_t* n_masked_left, pdllm_stream_t stream) {
+  if (!block_ids || !conf_out || !token_out || !transfer_out) return PDLLM_ERR_NULL;
+  if (n_seqs < 0 || block_len <= 0) return PDLLM_ERR_SHAPE;
+  if (last_logit && last_logit_stride < vocab) return PDLLM_ERR_STRIDE;
+  if (n_seqs == 0) return PDLLM_OK;
+  const int64_t n_rows = n_seqs * block_len;
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  const int st = vocab_launch(logits, logits_stride, last_logit, last_logit_stride, n_rows, block_len, vocab,
+                              shift ? 1 : 0, 2, nullptr, workspace, workspace_bytes, nullptr, nullptr, hs);
+  if (st != PDLLM_OK) return st;
+  const int ns = vocab_nsplit(n_rows, vocab);
+  long* pi = static_cast<long*>(workspace);
+  float* pm = reinterpret_cast<float*>(pi + n_rows * ns);
+  float* ps = pm + n_rows * ns;
+  hipLaunchKernelGGL(unmask_tail_kernel, dim3((unsigned)n_seqs), dim3(64), 0, hs, pm, ps, pi, ns,
+                     reinterpret_cast<long*>(block_ids), (long)block_len, (long)mask_token_id, threshold,
+                     conf_out, reinterpret_cast<long*>(token_out), transfer_out, n_masked_left);
   return launch_status();
 }

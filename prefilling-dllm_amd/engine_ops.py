@@ -167,6 +167,17 @@ def select_chunks_from_scores(scores: torch.Tensor, topk_chunks: int, keep_first
     return ops.topk_lowest_index(scores.contiguous(), k, sorted_ascending=True)
 
 
+def select_chunks_from_logits(logits: torch.Tensor, labels: torch.Tensor, topk_chunks: int,
+                              mean: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """score_chunk_self_information_engine (ENG:1098-1152) for all chunks of a draft round and the
+    ranking of select_chunks_by_engine (ENG:1199-1204) in one library call: logits
+    [n_chunks, n_labels, vocab] bf16 (the rows that predict the labels), labels [n_chunks, n_labels].
+    Returns (scores fp32 [n_chunks], selected chunk indices ascending)."""
+    n = int(logits.shape[0])
+    k = n if int(topk_chunks or 0) <= 0 else min(int(topk_chunks), n)
+    return ops.chunk_select_from_logits(logits, labels, k, mean=mean, sorted_ascending=True)
+
+
 # ------------------------------------------------------------------------------------------
 # token keep set (ENG:903-927)
 # ------------------------------------------------------------------------------------------
@@ -318,7 +329,6 @@ def denoise_unmask_step(logits: torch.Tensor, block_ids: torch.Tensor, *, mask_t
     uses shift=False.  Confidence = fp32 max-softmax, token = first argmax (_sample_tokens at
     temperature 0, ENG:1675-1681); transfer = most confident masked position plus every masked
     position with confidence >= threshold (ENG:2146-2157).  Returns (transfer mask, masked left)."""
-    n_seqs, block_len = block_ids.shape
-    conf, tok = ops.conf_argmax(logits, block_len, shift=shift, last_logit=last_context_logit)
-    return ops.threshold_unmask(conf.view(n_seqs, block_len), tok.view(n_seqs, block_len), block_ids,
-                                mask_token_id, threshold)
+    _, _, transfer, left = ops.denoise_unmask(logits, block_ids, mask_token_id, threshold, shift=shift,
+                                              last_logit=last_context_logit)
+    return transfer, left

@@ -445,6 +445,29 @@ def chunk_scores_from_logits(logits: torch.Tensor, labels: torch.Tensor, mean: b
     return out
 
 
+def chunk_select_from_logits(logits: torch.Tensor, labels: torch.Tensor, k: int, mean: bool = True,
+                             sorted_ascending: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """chunk_scores_from_logits followed by topk_lowest_index in one library call (two launches):
+    logits [n_chunks, n_labels, vocab] bf16, labels [n_chunks, n_labels] -> (scores fp32 [n_chunks],
+    indices int64 [min(k, n_chunks)]); fastdllm_engine.py:1148-1152 and 1199-1204."""
+    _need_cuda(logits, labels)
+    if logits.dtype != torch.bfloat16 or logits.dim() != 3 or not logits.is_contiguous():
+        raise ValueError("logits must be contiguous bf16 [n_chunks, n_labels, vocab]")
+    c, j, vocab = logits.shape
+    k = min(int(k), c)
+    if k <= 0:
+        raise ValueError("k must be positive")
+    labels = labels.to(torch.int64).reshape(c * j).contiguous()
+    scores = torch.empty(c, dtype=torch.float32, device=logits.device)
+    idx = torch.empty(k, dtype=torch.int64, device=logits.device)
+    need = lib.pdllm_vocab_workspace_bytes(c * j, vocab)
+    ws = _workspace(logits.device, int(need))
+    check(lib.pdllm_chunk_select(logits.data_ptr(), vocab, labels.data_ptr(), c, j, vocab, 1 if mean else 0, k,
+                                 1 if sorted_ascending else 0, _ptr(ws), 0 if ws is None else ws.numel(), None,
+                                 scores.data_ptr(), idx.data_ptr(), _stream(logits)), "chunk_select_from_logits")
+    return scores, idx
+
+
 def topk_lowest_index(scores: torch.Tensor, k: int, sorted_ascending: bool = True) -> torch.Tensor:
     """Top-k indices per row by (score desc, index asc); non-finite scores rank as -inf
     (fastdllm_engine.py:1199-1204)."""
@@ -648,6 +671,40 @@ def threshold_unmask(conf: torch.Tensor, token: torch.Tensor, block_ids: torch.T
                                      int(mask_token_id), float(threshold), transfer.data_ptr(), left.data_ptr(),
                                      _stream(block_ids)), "threshold_unmask")
     return transfer.view(torch.bool), left
+
+
+def denoise_unmask(logits: torch.Tensor, block_ids: torch.Tensor, mask_token_id: int, threshold: float,
+                   shift: bool = False, last_logit: Optional[torch.Tensor] = None
+                   ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """conf_argmax followed by threshold_unmask in one library call (two launches, no host sync):
+    bf16 logits [n_seqs*block_len, vocab], block_ids int64 [n_seqs, block_len] updated in place.
+    Returns (confidence fp32 [rows], token int64 [rows], transfer bool [n_seqs, block_len], masked left int32
+    [n_seqs]); fastdllm_engine.py:1647-1681 and 2146-2157."""
+    _need_cuda(logits, block_ids)
+    if logits.dtype != torch.bfloat16 or logits.stride(-1) != 1 or logits.dim() != 2:
+        raise ValueError("logits must be bf16 [rows, vocab]")
+    if block_ids.dtype != torch.int64 or not block_ids.is_contiguous() or block_ids.dim() != 2:
+        raise ValueError("block_ids must be contiguous int64 [n_seqs, block_len]")
+    rows, vocab = logits.shape
+    n_seqs, block_len = block_ids.shape
+    if rows != n_seqs * block_len:
+        raise ValueError("logits rows must equal n_seqs * block_len")
+    ll_ptr, ll_stride = None, 0
+    if last_logit is not None:
+        last_logit = last_logit.to(torch.bfloat16).reshape(n_seqs, vocab).contiguous()
+        ll_ptr, ll_stride = last_logit.data_ptr(), last_logit.stride(0)
+    dev = logits.device
+    conf = torch.empty(rows, dtype=torch.float32, device=dev)
+    tok = torch.empty(rows, dtype=torch.int64, device=dev)
+    transfer = torch.empty((n_seqs, block_len), dtype=torch.uint8, device=dev)
+    left = torch.empty(n_seqs, dtype=torch.int32, device=dev)
+    need = lib.pdllm_vocab_workspace_bytes(rows, vocab)
+    ws = _workspace(dev, int(need))
+    check(lib.pdllm_denoise_unmask(logits.data_ptr(), logits.stride(0), ll_ptr, ll_stride, n_seqs, block_len, vocab,
+                                   1 if shift else 0, block_ids.data_ptr(), int(mask_token_id), float(threshold),
+                                   _ptr(ws), 0 if ws is None else ws.numel(), conf.data_ptr(), tok.data_ptr(),
+                                   transfer.data_ptr(), left.data_ptr(), _stream(logits)), "denoise_unmask")
+    return conf, tok, transfer.view(torch.bool), left
 
 
 def rope_inplace(x: torch.Tensor, positions: torch.Tensor, cos_sin_cache: torch.Tensor) -> torch.Tensor:

@@ -31,6 +31,34 @@ def test_selfinfo_and_chunk_topk_config2(dev):
         assert srt[3] - srt[4] > 1e-3
 
 
+def test_chunk_select_single_call_equals_the_three_calls(dev):
+    """pdllm_chunk_select = selfinfo_logprob + chunk_score_reduce + topk_lowest_index, bit for bit, and the
+    oracle's selection; also with tied and non-finite chunk scores (labels outside the vocabulary give -inf)."""
+    ops = _ops()
+    logits, labels = configs.draft_logits(seed=4)
+    dl, dlab = logits.to(dev), labels.to(dev)
+    for mean in (False, True):
+        for asc in (True, False):
+            sc, idx = ops.chunk_select_from_logits(dl, dlab, 4, mean=mean, sorted_ascending=asc)
+            sc3 = ops.chunk_scores_from_logits(dl, dlab, mean=mean)
+            assert torch.equal(sc, sc3)
+            assert torch.equal(idx, ops.topk_lowest_index(sc3, 4, sorted_ascending=asc))
+            ref = ref_ops.chunk_scores(logits, labels, mean=mean)
+            assert idx.cpu().tolist() == ref_ops.topk_lowest_index(ref.tolist(), 4, sorted_ascending=asc)
+    # ties and -inf: chunks 1 and 2 are identical rows, chunk 3 has a label outside the vocabulary
+    gen = torch.Generator().manual_seed(9)
+    small = (torch.randn(6, 2, 5000, generator=gen) * 2).to(torch.bfloat16)
+    small[2] = small[1]
+    lab = torch.randint(0, 5000, (6, 2), generator=gen)
+    lab[2] = lab[1]
+    lab[3, 0] = -1
+    for k in range(1, 7):
+        sc, idx = ops.chunk_select_from_logits(small.to(dev), lab.to(dev), k, mean=False)
+        assert torch.isinf(sc[3]) and sc[3] < 0 and sc[1] == sc[2]
+        assert idx.cpu().tolist() == ref_ops.topk_lowest_index(sc.cpu().tolist(), k), k
+        assert torch.equal(idx, ops.topk_lowest_index(sc, k))
+
+
 def test_selfinfo_ragged_vocab_and_bad_label(dev):
     gen = torch.Generator().manual_seed(2)
     logits = (torch.randn(5, 1003, generator=gen) * 3).to(torch.bfloat16)  # rows not 16-byte aligned
@@ -180,6 +208,31 @@ def test_unmask_with_dream_shift(dev):
     conf2, tok2 = _ops().conf_argmax(logits.to(dev), L, shift=True)
     sh = ref_ops.shift_logits(logits[:L], None)
     assert torch.equal(tok2[:L].cpu(), ref_ops.sample_tokens(sh)[1])
+
+
+def test_denoise_unmask_single_call_equals_the_two_calls(dev):
+    """pdllm_denoise_unmask = conf_argmax + threshold_unmask, bit for bit, with the Dream shift, a last
+    context logit, partly decoded blocks and a block with nothing left to unmask."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(14)
+    vocab, L, n_seqs, mask_id = 9000, 32, 3, 8999
+    logits = (torch.randn(n_seqs * L, vocab, generator=gen) * 2).to(torch.bfloat16)
+    rows = torch.randperm(n_seqs * L, generator=gen)[:40]
+    logits[rows, torch.randint(0, vocab - 1, (40,), generator=gen)] = 20.0   # confident rows
+    last = (torch.randn(n_seqs, vocab, generator=gen) * 2).to(torch.bfloat16)
+    block = torch.full((n_seqs, L), mask_id, dtype=torch.int64)
+    block[0, :7] = 5
+    block[2] = 6                                                               # nothing masked
+    for shift, ll in ((False, None), (True, None), (True, last)):
+        a_ids, b_ids = block.clone().to(dev), block.clone().to(dev)
+        lld = None if ll is None else ll.to(dev)
+        conf, tok, tr, left = ops.denoise_unmask(logits.to(dev), a_ids, mask_id, 0.9, shift=shift, last_logit=lld)
+        conf2, tok2 = ops.conf_argmax(logits.to(dev), L, shift=shift, last_logit=lld)
+        tr2, left2 = ops.threshold_unmask(conf2.view(n_seqs, L), tok2.view(n_seqs, L), b_ids, mask_id, 0.9)
+        assert torch.equal(conf, conf2) and torch.equal(tok, tok2)
+        assert torch.equal(tr, tr2) and torch.equal(left, left2) and torch.equal(a_ids, b_ids)
+        assert int(left[2]) == 0 and not bool(tr[2].any())
+        assert int(tr[0, :7].sum()) == 0 and int(tr[0].sum()) >= 1
 
 
 def test_argmax_first_index_on_ties(dev):
