@@ -282,6 +282,16 @@ int pdllm_kv_scatter(void* cache, const int32_t* page_ids, int64_t n_page_ids, i
                      int64_t n_tokens, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
                      int64_t n_pages, int32_t elem_bytes, const void* src, pdllm_stream_t stream);
 
+/* Replaces the per-layer advanced-indexing copies of make_pd_record_from_remote_engine
+ * (ENG:845-859) for two unified caches [planes, n_pages, page_size, Hkv, d] (plane = K/V x layer)
+ * of the same page geometry: dst[plane][dst_page_ids[i]] = src[plane][src_page_ids[i]] for all
+ * planes in one launch, page-granular (the tokens of a last, partly filled page travel with their
+ * page).  Strides and page_bytes in bytes, multiples of 16; page ids outside a cache are skipped. */
+int pdllm_kv_copy_pages(const void* src_cache, void* dst_cache, const int32_t* src_page_ids,
+                        const int32_t* dst_page_ids, int64_t n_copy, int64_t page_bytes, int64_t n_planes,
+                        int64_t src_plane_stride_bytes, int64_t dst_plane_stride_bytes,
+                        int64_t src_n_pages, int64_t dst_n_pages, pdllm_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Confidence-threshold unmasking                                             *
  * ------------------------------------------------------------------------- */

@@ -172,6 +172,31 @@ __global__ __launch_bounds__(256) void kv_scatter_kernel(
   cache[slot * per_tok + rem] = src[idx];
 }
 
+// whole pages between two caches, all planes (K/V x layer) in one launch:
+// dst[plane][dst_page_ids[i]] = src[plane][src_page_ids[i]]; pages outside either cache are skipped
+__global__ __launch_bounds__(256) void kv_copy_pages_kernel(
+    const uint4* __restrict__ src, uint4* __restrict__ dst, const int* __restrict__ src_page_ids,
+    const int* __restrict__ dst_page_ids, long page16, long src_plane16, long dst_plane16, long src_n_pages,
+    long dst_n_pages, int parts) {
+  const long i = blockIdx.x / parts;
+  const int part = blockIdx.x - (int)i * parts;
+  const long plane = blockIdx.y;
+  const long sp = src_page_ids[i], dp = dst_page_ids[i];
+  if (sp < 0 || sp >= src_n_pages || dp < 0 || dp >= dst_n_pages) return;
+  const uint4* s = src + plane * src_plane16 + sp * page16;
+  uint4* d = dst + plane * dst_plane16 + dp * page16;
+  const long seg = (page16 + parts - 1) / parts;
+  const long begin = (long)part * seg;
+  long end = begin + seg;
+  end = end < page16 ? end : page16;
+  long c = begin + threadIdx.x;
+  for (; c + 3 * 256 < end; c += 4 * 256) {  // four 16-byte loads in flight per lane
+    const uint4 a0 = s[c], a1 = s[c + 256], a2 = s[c + 512], a3 = s[c + 768];
+    d[c] = a0; d[c + 256] = a1; d[c + 512] = a2; d[c + 768] = a3;
+  }
+  for (; c < end; c += 256) d[c] = s[c];
+}
+
 static int ilog2_exact_l(long v) {
   if (v <= 0 || (v & (v - 1))) return -1;
   int s = 0;
@@ -319,5 +344,29 @@ extern "C" int pdllm_kv_scatter(void* cache, const int32_t* page_ids, int64_t n_
                      static_cast<hipStream_t>(stream), static_cast<uint4*>(cache), page_ids,
                      (long)n_page_ids, (long)dst_start, (long)n_tokens, per_tok, shift, (long)n_pages,
                      static_cast<const uint4*>(src));
+  return launch_status();
+}
+
+extern "C" int pdllm_kv_copy_pages(const void* src_cache, void* dst_cache, const int32_t* src_page_ids,
+                                   const int32_t* dst_page_ids, int64_t n_copy, int64_t page_bytes,
+                                   int64_t n_planes, int64_t src_plane_stride_bytes,
+                                   int64_t dst_plane_stride_bytes, int64_t src_n_pages, int64_t dst_n_pages,
+                                   pdllm_stream_t stream) {
+  if (!src_cache || !dst_cache || !src_page_ids || !dst_page_ids) return PDLLM_ERR_NULL;
+  if (n_copy < 0 || page_bytes <= 0 || n_planes <= 0 || n_planes > 65535 || src_n_pages <= 0 || dst_n_pages <= 0)
+    return PDLLM_ERR_SHAPE;
+  if (page_bytes % 16 || src_plane_stride_bytes % 16 || dst_plane_stride_bytes % 16 ||
+      src_plane_stride_bytes < src_n_pages * page_bytes || dst_plane_stride_bytes < dst_n_pages * page_bytes)
+    return PDLLM_ERR_STRIDE;
+  if (!aligned16(src_cache) || !aligned16(dst_cache)) return PDLLM_ERR_STRIDE;
+  if (n_copy == 0) return PDLLM_OK;
+  // about 64 KB per workgroup
+  int parts = (int)((page_bytes + 65535) / 65536);
+  if (n_copy * parts > 0x7fffffffL) return PDLLM_ERR_SHAPE;
+  hipLaunchKernelGGL(kv_copy_pages_kernel, dim3((unsigned)(n_copy * parts), (unsigned)n_planes), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint4*>(src_cache),
+                     static_cast<uint4*>(dst_cache), src_page_ids, dst_page_ids, (long)(page_bytes / 16),
+                     (long)(src_plane_stride_bytes / 16), (long)(dst_plane_stride_bytes / 16), (long)src_n_pages,
+                     (long)dst_n_pages, parts);
   return launch_status();
 }

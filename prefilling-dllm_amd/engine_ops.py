@@ -293,6 +293,82 @@ def snapshot_pd_record_kv(kv_cache: torch.Tensor, record: DreamPrefillRecord, *,
                            last_context_logit=None if ll is None else ll.to(device))
 
 
+def _allocate_record_pages(allocator: PrefixPageAllocator, prompt_len: int, decode_len: int,
+                           page_size: int) -> Tuple[List[int], List[int]]:
+    """Pages for a record on the decode side: evict unreferenced cached prefixes until both lists fit
+    (ENG:746-751), then take the prompt pages and the block pages."""
+    n_prompt = math.ceil(prompt_len / page_size)
+    n_block = math.ceil(decode_len / page_size)
+    while allocator.num_free_pages < n_prompt + n_block:
+        if not allocator.evict_one():
+            break
+    return allocator.allocate_pages(n_prompt), allocator.allocate_pages(n_block)
+
+
+def _decode_side_record(source: DreamPrefillRecord, prompt_page_ids: List[int], block_page_ids: List[int],
+                        last_context_logit: Optional[torch.Tensor]) -> DreamPrefillRecord:
+    return DreamPrefillRecord(
+        prompt_ids=list(source.prompt_ids), prompt_positions=list(source.prompt_positions),
+        suffix_positions=list(source.suffix_positions), prompt_len=source.prompt_len,
+        full_prompt_len=source.full_prompt_len, decode_len=source.decode_len, prompt_page_ids=prompt_page_ids,
+        block_page_ids=block_page_ids, first_token_id=source.first_token_id, last_context_logit=last_context_logit,
+        decode_delta_state=source.decode_delta_state, owns_prompt_pages=True, cached_prefix=None,
+        kv_mode=source.kv_mode)
+
+
+def make_pd_record_from_kv_snapshot(kv_cache: torch.Tensor, allocator: PrefixPageAllocator,
+                                    source: DreamPrefillRecord, snapshot: DreamKVSnapshot, *,
+                                    page_size: int = PAGE_SIZE) -> DreamPrefillRecord:
+    """make_pd_record_from_kv_snapshot (ENG:728-781): allocate local pages, load the snapshot into them
+    and return the record the decode side works on; the same three consistency checks."""
+    if snapshot.page_size != page_size:
+        raise ValueError(f"PD KV snapshot page_size mismatch: snapshot={snapshot.page_size}, engine={page_size}")
+    if snapshot.prompt_len != source.prompt_len:
+        raise ValueError(f"PD KV snapshot prompt_len mismatch: snapshot={snapshot.prompt_len}, "
+                         f"source={source.prompt_len}")
+    if snapshot.kv_mode != source.kv_mode:
+        raise ValueError(f"PD KV snapshot mode mismatch: snapshot={snapshot.kv_mode}, source={source.kv_mode}")
+    prompt_pages, block_pages = _allocate_record_pages(allocator, source.prompt_len, source.decode_len, page_size)
+    load_prompt_cache_per_layer(kv_cache, prompt_pages, source.prompt_len, snapshot.k_by_layer, snapshot.v_by_layer)
+    ll = snapshot.last_context_logit
+    if ll is not None:
+        ll = ll.to(device=kv_cache.device).contiguous()
+    return _decode_side_record(source, prompt_pages, block_pages, ll)
+
+
+def make_pd_record_from_remote_cache(src_kv_cache: torch.Tensor, dst_kv_cache: torch.Tensor,
+                                     allocator: PrefixPageAllocator, source: DreamPrefillRecord, *,
+                                     page_size: int = PAGE_SIZE) -> DreamPrefillRecord:
+    """make_pd_record_from_remote_engine (ENG:800-881) for two caches on this GPU: the prompt KV moves
+    page by page, all layers in one launch, instead of one gather and one indexed write per layer."""
+    if int(src_kv_cache.shape[3]) != page_size or int(dst_kv_cache.shape[3]) != page_size:
+        raise ValueError(f"remote-engine PD page_size mismatch: source={int(src_kv_cache.shape[3])}, "
+                         f"target={int(dst_kv_cache.shape[3])}")
+    if int(src_kv_cache.shape[1]) != int(dst_kv_cache.shape[1]):
+        raise ValueError(f"remote-engine PD layer mismatch: source={int(src_kv_cache.shape[1])}, "
+                         f"target={int(dst_kv_cache.shape[1])}")
+    prompt_pages, block_pages = _allocate_record_pages(allocator, source.prompt_len, source.decode_len, page_size)
+    n = len(prompt_pages)
+    dev = dst_kv_cache.device
+    ops.kv_copy_pages(src_kv_cache, dst_kv_cache,
+                      torch.as_tensor(list(source.prompt_page_ids)[:n], dtype=torch.int32, device=dev),
+                      torch.as_tensor(prompt_pages, dtype=torch.int32, device=dev))
+    ll = source.last_context_logit
+    if ll is not None:
+        ll = ll.to(device=dev).contiguous()
+    return _decode_side_record(source, prompt_pages, block_pages, ll)
+
+
+def release_pd_record(allocator: PrefixPageAllocator, record: DreamPrefillRecord) -> None:
+    """release_pd_record (ENG:2192-2198): block pages always go back, prompt pages when the record owns
+    them, and a shared prefix loses one reference."""
+    allocator.release_pages(record.block_page_ids)
+    if record.owns_prompt_pages:
+        allocator.release_pages(record.prompt_page_ids)
+    if record.cached_prefix is not None:
+        record.cached_prefix.ref_count -= 1
+
+
 def copy_chunk_local_kv_to_prompt_pages(kv_cache: torch.Tensor, *, src_page_ids: Sequence[int],
                                         dst_page_ids: Sequence[int], src_chunk_start: int, dst_start: int,
                                         keep_indices_per_layer_per_head: Sequence[torch.Tensor]) -> int:

@@ -625,6 +625,32 @@ def kv_scatter(layer_cache: torch.Tensor, page_ids: torch.Tensor, src: torch.Ten
                                _stream(layer_cache)), "kv_scatter")
 
 
+def kv_copy_pages(src_kv_cache: torch.Tensor, dst_kv_cache: torch.Tensor, src_page_ids: torch.Tensor,
+                  dst_page_ids: torch.Tensor) -> None:
+    """dst[:, :, dst_page_ids[i]] = src[:, :, src_page_ids[i]] for two unified caches
+    [2, layers, n_pages, page_size, Hkv, d] of the same page geometry and dtype, all layers in one
+    launch (the page-granular form of the copies in fastdllm_engine.py:845-859)."""
+    _need_cuda(src_kv_cache, dst_kv_cache, src_page_ids, dst_page_ids)
+    if src_kv_cache.dim() != 6 or dst_kv_cache.dim() != 6 or not src_kv_cache.is_contiguous() or \
+            not dst_kv_cache.is_contiguous():
+        raise ValueError("caches must be contiguous [2, layers, n_pages, page_size, Hkv, d]")
+    if src_kv_cache.shape[:2] != dst_kv_cache.shape[:2] or src_kv_cache.shape[3:] != dst_kv_cache.shape[3:] or \
+            src_kv_cache.dtype != dst_kv_cache.dtype:
+        raise ValueError("source and destination caches differ in layers, page geometry or dtype")
+    if src_page_ids.numel() != dst_page_ids.numel():
+        raise ValueError("page id lists differ in length")
+    sp = src_page_ids.to(torch.int32).contiguous()
+    dp = dst_page_ids.to(torch.int32).contiguous()
+    planes = src_kv_cache.shape[0] * src_kv_cache.shape[1]
+    page_bytes = src_kv_cache.stride(2) * src_kv_cache.element_size()
+    check(lib.pdllm_kv_copy_pages(src_kv_cache.data_ptr(), dst_kv_cache.data_ptr(), sp.data_ptr(), dp.data_ptr(),
+                                  sp.numel(), page_bytes, planes,
+                                  src_kv_cache.stride(1) * src_kv_cache.element_size(),
+                                  dst_kv_cache.stride(1) * dst_kv_cache.element_size(),
+                                  src_kv_cache.shape[2], dst_kv_cache.shape[2], _stream(dst_kv_cache)),
+          "kv_copy_pages")
+
+
 # ----------------------------------------------------------------------------------------
 # confidence / unmask / rope
 # ----------------------------------------------------------------------------------------

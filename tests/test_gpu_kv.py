@@ -122,6 +122,68 @@ def test_gather_scatter_roundtrip_and_snapshot(dev):
     assert torch.equal(cache2.cpu(), ref2)
 
 
+def test_pd_handoff_snapshot_and_page_copy(dev):
+    """The prefill/decode hand-off both ways the reference has it (fastdllm_engine.py:700-881): through a host
+    snapshot loaded into freshly allocated pages, and cache to cache page by page.  Either way the decode side
+    reads back exactly the prompt KV of the prefill side; pages it did not receive stay untouched."""
+    from prefilling_dllm_amd import engine_ops as eo
+    ops = _ops()
+    gen = torch.Generator().manual_seed(8)
+    L, n_pages, P, Hkv, d = 3, 10, 256, 4, 128
+    src = torch.randn(2, L, n_pages, P, Hkv, d, generator=gen).to(torch.bfloat16).to(dev)
+    prompt_len, decode_len = 700, 96
+    src_pages = [7, 2, 5]
+    rec = eo.DreamPrefillRecord(prompt_ids=list(range(prompt_len)), prompt_positions=list(range(prompt_len)),
+                                suffix_positions=list(range(prompt_len, prompt_len + decode_len)),
+                                prompt_len=prompt_len, full_prompt_len=prompt_len, decode_len=decode_len,
+                                prompt_page_ids=src_pages, block_page_ids=[9], first_token_id=1,
+                                last_context_logit=torch.arange(8, dtype=torch.float32, device=dev),
+                                decode_delta_state=None, owns_prompt_pages=True)
+    want_k, want_v = eo.snapshot_prompt_cache_per_layer(src, src_pages, prompt_len)
+    for l in range(L):
+        idx = torch.arange(prompt_len)
+        assert torch.equal(want_k[l].cpu(), ref_ops.gather_tokens(src[0, l].cpu(), torch.tensor(src_pages), idx))
+
+    # (1) host snapshot -> another engine's cache
+    snap = eo.snapshot_pd_record_kv(src, rec, device="cpu")
+    assert snap.k_by_layer[0].device.type == "cpu" and tuple(snap.k_by_layer[0].shape) == (prompt_len, Hkv, d)
+    dst = torch.zeros_like(src)
+    alloc = eo.PrefixPageAllocator(n_pages, P)
+    alloc.allocate_pages(2)                                     # pages 0, 1 are taken by someone else
+    rec2 = eo.make_pd_record_from_kv_snapshot(dst, alloc, rec, snap)
+    assert rec2.prompt_page_ids == [2, 3, 4] and rec2.block_page_ids == [5] and rec2.owns_prompt_pages
+    got_k, got_v = eo.snapshot_prompt_cache_per_layer(dst, rec2.prompt_page_ids, prompt_len)
+    for l in range(L):
+        assert torch.equal(got_k[l], want_k[l]) and torch.equal(got_v[l], want_v[l])
+    assert int(dst[:, :, [0, 1, 5, 6, 7, 8, 9]].abs().sum()) == 0
+    assert torch.equal(rec2.last_context_logit, rec.last_context_logit)
+    with pytest.raises(ValueError, match="page_size mismatch"):
+        eo.make_pd_record_from_kv_snapshot(dst, alloc, rec, snap, page_size=128)
+    snap.prompt_len += 1
+    with pytest.raises(ValueError, match="prompt_len mismatch"):
+        eo.make_pd_record_from_kv_snapshot(dst, alloc, rec, snap)
+    eo.release_pd_record(alloc, rec2)
+    assert alloc.num_free_pages == n_pages - 2
+
+    # (2) cache to cache, whole pages, all layers in one launch
+    dst2 = torch.zeros_like(src)
+    alloc2 = eo.PrefixPageAllocator(n_pages, P)
+    alloc2.allocate_pages(4)
+    rec3 = eo.make_pd_record_from_remote_cache(src, dst2, alloc2, rec)
+    assert rec3.prompt_page_ids == [4, 5, 6]
+    for a, b in zip(src_pages, rec3.prompt_page_ids):
+        assert torch.equal(dst2[:, :, b], src[:, :, a])
+    assert int(dst2[:, :, [0, 1, 2, 3, 7, 8, 9]].abs().sum()) == 0
+    got_k, got_v = eo.snapshot_prompt_cache_per_layer(dst2, rec3.prompt_page_ids, prompt_len)
+    for l in range(L):
+        assert torch.equal(got_k[l], want_k[l]) and torch.equal(got_v[l], want_v[l])
+    # page ids outside either cache are skipped, not written
+    ops.kv_copy_pages(src, dst2, torch.tensor([1, 99], dtype=torch.int32, device=dev),
+                      torch.tensor([-1, 0], dtype=torch.int32, device=dev))
+    torch.cuda.synchronize()
+    assert int(dst2[:, :, 0].abs().sum()) == 0
+
+
 def test_per_head_compaction_matches_reference_order(dev):
     """fastdllm_engine.py:607-638: gather with per-head keep lists, rewrite into the first slots."""
     gen = torch.Generator().manual_seed(5)
