@@ -336,6 +336,19 @@ int pdllm_rope_inplace(void* x, int64_t x_stride, const int64_t* positions,
                        const float* cos_sin_cache, int64_t max_positions, int64_t n_tokens,
                        int32_t n_heads, int32_t head_dim, pdllm_stream_t stream);
 
+/* RotaryEmbedding.forward on Q and K (layers/rotary_embedding.py:39-65) and the paged store of the
+ * rotated K and of V (OPS/kv_cache_kernels.py:150-172) in one launch, the order the reference's
+ * attention layer runs them in (rotary, then Attention.forward stores K/V, attention_v4.py:316-335).
+ * q [n_tokens, num_q_heads, d] and k [n_tokens, num_kv_heads, d] bf16 are rotated in place; with
+ * slot_mapping != NULL, cache row slot_mapping[t] of the unified bf16 caches receives the rotated K
+ * and V of token t (slots < 0 or >= n_slots: not stored).  Same bits as pdllm_rope_inplace on q and
+ * k followed by pdllm_kv_store.  head_dim % 16 == 0, strides in elements and multiples of 8. */
+int pdllm_rope_qk_store(void* q, int64_t q_stride, int32_t num_q_heads, void* k, int64_t k_stride,
+                        const void* v, int64_t v_stride, int32_t num_kv_heads, int32_t head_dim,
+                        const int64_t* positions, const float* cos_sin_cache, int64_t max_positions,
+                        int64_t n_tokens, void* k_cache, void* v_cache, const int32_t* slot_mapping,
+                        int64_t n_slots, pdllm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -330,6 +330,15 @@ __global__ __launch_bounds__(64) void threshold_unmask_kernel(
   if (lane == 0 && n_left) n_left[b] = n_masked - moved;
 }
 
+// one rotation in fp32 with every product and sum rounded on its own, as the unfused torch expression
+// x1 * cos - x2 * sin, x2 * cos + x1 * sin evaluates (no fused multiply-add)
+__device__ __forceinline__ void rope_pair(float x1, float x2, float c, float s, float& y1, float& y2) {
+#pragma clang fp contract(off)
+  const float a = x1 * c, b = x2 * s, e = x2 * c, f = x1 * s;
+  y1 = a - b;
+  y2 = e + f;
+}
+
 // neox rotary embedding in place: x [n_tokens, n_heads, d] bf16
 __global__ __launch_bounds__(256) void rope_kernel(__bf16* __restrict__ x, long x_stride,
                                                    const long* __restrict__ positions,
@@ -348,11 +357,64 @@ __global__ __launch_bounds__(256) void rope_kernel(__bf16* __restrict__ x, long 
   const float s = cos_sin[pos * head_dim + half + i];
   __bf16* p = x + t * x_stride + (long)hd * head_dim;
   const float x1 = (float)p[i], x2 = (float)p[i + half];
-  // fp32 products rounded separately, as the unfused torch expression
-  const float y1 = __fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s));
-  const float y2 = __fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, s));
+  float y1, y2;
+  rope_pair(x1, x2, c, s, y1, y2);
   p[i] = (__bf16)y1;
   p[i + half] = (__bf16)y2;
+}
+
+// Rotary embedding of Q and K in place and the paged store of the rotated K and of V in one pass:
+// what rope_kernel on Q, rope_kernel on K and the store kernel do one after the other, with K read
+// once.  A thread rotates 8 + 8 elements of one head (16-byte loads) or copies 16 bytes of a V row.
+__global__ __launch_bounds__(256) void rope_qk_store_kernel(
+    __bf16* __restrict__ q, long q_stride, int Hq, __bf16* __restrict__ k, long k_stride,
+    const __bf16* __restrict__ v, long v_stride, int Hkv, int head_dim, const long* __restrict__ positions,
+    const float* __restrict__ cos_sin, long max_pos, long n_tokens, __bf16* __restrict__ k_cache,
+    __bf16* __restrict__ v_cache, const int* __restrict__ slots, long n_slots) {
+  const int half = head_dim / 2;
+  const int hc = half / 8;  // 8-element groups per half head
+  const int per_q = Hq * hc, per_k = Hkv * hc, per_v = Hkv * head_dim / 8;
+  const long per_tok = per_q + per_k + per_v;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const long t = idx / per_tok;
+  if (t >= n_tokens) return;
+  const int r = (int)(idx - t * per_tok);
+  long slot = slots ? (long)slots[t] : -1;
+  if (slot >= n_slots) slot = -1;
+  const long row = (long)Hkv * head_dim;
+  if (r >= per_q + per_k) {
+    if (slot >= 0) {
+      const int c = r - per_q - per_k;
+      *reinterpret_cast<uint4*>(v_cache + slot * row + 8 * c) = *reinterpret_cast<const uint4*>(v + t * v_stride + 8 * c);
+    }
+    return;
+  }
+  const bool is_k = r >= per_q;
+  const int rr = is_k ? r - per_q : r;
+  const int hd = rr / hc, g = rr - hd * hc;
+  __bf16* p = (is_k ? k + t * k_stride : q + t * q_stride) + (long)hd * head_dim + 8 * g;
+  bf16x8 lo = *reinterpret_cast<const bf16x8*>(p);
+  bf16x8 hi = *reinterpret_cast<const bf16x8*>(p + half);
+  const long pos = positions[t];
+  if (pos >= 0 && pos < max_pos) {
+    const float* cs = cos_sin + pos * head_dim + 8 * g;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float c = cs[j], sn = cs[half + j];
+      const float x1 = (float)lo[j], x2 = (float)hi[j];
+      float y1, y2;
+      rope_pair(x1, x2, c, sn, y1, y2);
+      lo[j] = (__bf16)y1;
+      hi[j] = (__bf16)y2;
+    }
+    *reinterpret_cast<bf16x8*>(p) = lo;
+    *reinterpret_cast<bf16x8*>(p + half) = hi;
+  }
+  if (is_k && slot >= 0) {
+    __bf16* dst = k_cache + slot * row + (long)hd * head_dim + 8 * g;
+    *reinterpret_cast<bf16x8*>(dst) = lo;
+    *reinterpret_cast<bf16x8*>(dst + half) = hi;
+  }
 }
 
 static int vocab_nsplit(long n_rows, long vocab) {
@@ -514,5 +576,34 @@ extern "C" int pdllm_denoise_unmask(const void* logits, int64_t logits_stride, c
   hipLaunchKernelGGL(unmask_tail_kernel, dim3((unsigned)n_seqs), dim3(64), 0, hs, pm, ps, pi, ns,
                      reinterpret_cast<long*>(block_ids), (long)block_len, (long)mask_token_id, threshold,
                      conf_out, reinterpret_cast<long*>(token_out), transfer_out, n_masked_left);
+  return launch_status();
+}
+
+extern "C" int pdllm_rope_qk_store(void* q, int64_t q_stride, int32_t num_q_heads, void* k, int64_t k_stride,
+                                   const void* v, int64_t v_stride, int32_t num_kv_heads, int32_t head_dim,
+                                   const int64_t* positions, const float* cos_sin_cache, int64_t max_positions,
+                                   int64_t n_tokens, void* k_cache, void* v_cache, const int32_t* slot_mapping,
+                                   int64_t n_slots, pdllm_stream_t stream) {
+  if (!q || !k || !positions || !cos_sin_cache) return PDLLM_ERR_NULL;
+  if (slot_mapping && (!v || !k_cache || !v_cache)) return PDLLM_ERR_NULL;
+  if (n_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || head_dim % 16 || max_positions <= 0 ||
+      n_slots < 0)
+    return PDLLM_ERR_SHAPE;
+  if (q_stride < (int64_t)num_q_heads * head_dim || k_stride < (int64_t)num_kv_heads * head_dim || q_stride % 8 ||
+      k_stride % 8)
+    return PDLLM_ERR_STRIDE;
+  if (slot_mapping && (v_stride < (int64_t)num_kv_heads * head_dim || v_stride % 8)) return PDLLM_ERR_STRIDE;
+  if (((uintptr_t)q % 16) || ((uintptr_t)k % 16) || ((uintptr_t)cos_sin_cache % 4)) return PDLLM_ERR_STRIDE;
+  if (slot_mapping && (((uintptr_t)v % 16) || ((uintptr_t)k_cache % 16) || ((uintptr_t)v_cache % 16))) return PDLLM_ERR_STRIDE;
+  if (n_tokens == 0) return PDLLM_OK;
+  const long per_tok = (long)(num_q_heads + num_kv_heads) * (head_dim / 16) + (long)num_kv_heads * head_dim / 8;
+  const long total = n_tokens * per_tok;
+  if ((total + 255) / 256 > 0x7fffffffL) return PDLLM_ERR_SHAPE;
+  hipLaunchKernelGGL(rope_qk_store_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<__bf16*>(q), (long)q_stride, num_q_heads,
+                     static_cast<__bf16*>(k), (long)k_stride, static_cast<const __bf16*>(v), (long)v_stride,
+                     num_kv_heads, head_dim, reinterpret_cast<const long*>(positions), cos_sin_cache,
+                     (long)max_positions, (long)n_tokens, static_cast<__bf16*>(k_cache),
+                     static_cast<__bf16*>(v_cache), slot_mapping, (long)n_slots);
   return launch_status();
 }

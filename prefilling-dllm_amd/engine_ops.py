@@ -394,6 +394,57 @@ def copy_chunk_local_kv_to_prompt_pages(kv_cache: torch.Tensor, *, src_page_ids:
 
 
 # ------------------------------------------------------------------------------------------
+# rotary positions of chunks and queries (prefilling_dllm_eval/fastdllm_parallelcomp.py:919-948)
+# ------------------------------------------------------------------------------------------
+
+def chunk_rope_start(mode: str, prefix_len: int, chunk_order: int, chunk_index: int, chunk_size: int) -> int:
+    """First rotary position of a chunk (_chunk_rope_start): "reuse" puts every chunk right behind the
+    prefix, "continuous" lines the chunks up in the order they are processed, "absolute" by their index in
+    the document."""
+    step = max(1, int(chunk_size))
+    if mode == "reuse":
+        return int(prefix_len)
+    if mode == "continuous":
+        return int(prefix_len) + int(chunk_order) * step
+    if mode == "absolute":
+        return int(prefix_len) + int(chunk_index) * step
+    raise ValueError(f"Unsupported chunk_position_mode: {mode}")
+
+
+def chunk_query_rope_start(mode: str, prefix_len: int, chunk_start: int, chunk_len: int, chunk_size: int) -> int:
+    """First rotary position of the query appended to a chunk while it is scored (_chunk_query_rope_start)."""
+    if mode == "after_reused_window":
+        return int(prefix_len) + max(1, int(chunk_size))
+    if mode == "after_chunk":
+        return int(chunk_start) + int(chunk_len)
+    raise ValueError(f"Unsupported chunk_query_position_mode: {mode}")
+
+
+def final_query_rope_start(mode: str, prefix_len: int, cache_positions: Sequence[int], selected_count: int,
+                           chunk_size: int) -> int:
+    """First rotary position of the query + response block of the decode (_final_query_rope_start)."""
+    if mode == "after_reused_window":
+        return int(prefix_len) + max(1, int(chunk_size))
+    if mode == "after_selected_chunks":
+        return int(prefix_len) + int(selected_count) * max(1, int(chunk_size))
+    if mode == "after_cache":
+        return (max(cache_positions) + 1) if len(cache_positions) else int(prefix_len)
+    raise ValueError(f"Unsupported query_position_mode: {mode}")
+
+
+def chunk_positions(mode: str, prefix_len: int, chunk_lens: Sequence[int], chunk_indices: Sequence[int],
+                    chunk_size: int, device=None) -> torch.Tensor:
+    """Rotary positions of a packed batch of chunks (int64 [sum(chunk_lens)]): chunk j, the j-th processed
+    and chunk_indices[j]-th of the document, gets chunk_rope_start(...) + 0 .. len-1."""
+    out = []
+    for order, (n, ci) in enumerate(zip(chunk_lens, chunk_indices)):
+        s0 = chunk_rope_start(mode, prefix_len, order, ci, chunk_size)
+        out.append(torch.arange(s0, s0 + int(n), dtype=torch.int64))
+    pos = torch.cat(out) if out else torch.empty(0, dtype=torch.int64)
+    return pos if device is None else pos.to(device)
+
+
+# ------------------------------------------------------------------------------------------
 # one denoise step after the model forward (ENG:2143-2157), no host synchronisation
 # ------------------------------------------------------------------------------------------
 

@@ -744,3 +744,34 @@ def rope_inplace(x: torch.Tensor, positions: torch.Tensor, cos_sin_cache: torch.
     check(lib.pdllm_rope_inplace(x.data_ptr(), x.stride(0), positions.data_ptr(), cs.data_ptr(), cs.shape[0], n, h,
                                  d, _stream(x)), "rope_inplace")
     return x
+
+
+def rope_qk_store(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], positions: torch.Tensor,
+                  cos_sin_cache: torch.Tensor, k_cache: Optional[torch.Tensor] = None,
+                  v_cache: Optional[torch.Tensor] = None, slot_mapping: Optional[torch.Tensor] = None) -> None:
+    """rope_inplace on q and k and store_kvcache_unified_layout of (rotated k, v) in one launch
+    (layers/rotary_embedding.py:39-65 then kv_cache_kernels.py:150-172).  q [n, Hq, d], k / v [n, Hkv, d]
+    bf16; without slot_mapping only the rotation is done."""
+    _need_cuda(q, k, positions, cos_sin_cache)
+    n, hq, d = q.shape
+    hkv = k.shape[1]
+    for name, x in (("q", q), ("k", k)) + ((("v", v),) if v is not None else ()):
+        if x.dtype != torch.bfloat16 or x.stride(-1) != 1 or x.stride(1) != d or x.shape[0] != n or x.shape[2] != d:
+            raise ValueError(f"{name} must be bf16 [tokens, heads, d] with contiguous heads")
+    positions = positions.to(torch.int64).contiguous()
+    cs = cos_sin_cache.float().contiguous()
+    slots_ptr, n_slots, kc_ptr, vc_ptr, v_ptr, v_stride = None, 0, None, None, None, 0
+    if slot_mapping is not None:
+        if v is None or k_cache is None or v_cache is None:
+            raise ValueError("slot_mapping needs v and both caches")
+        if not k_cache.is_contiguous() or not v_cache.is_contiguous() or k_cache.dtype != torch.bfloat16 or \
+                tuple(k_cache.shape[2:]) != (hkv, d):
+            raise ValueError("the fused store needs contiguous bf16 unified caches [pages, page_size, Hkv, d]")
+        slot_mapping = slot_mapping.to(torch.int32).contiguous()
+        if slot_mapping.numel() != n:
+            raise ValueError("slot_mapping must have one entry per token")
+        slots_ptr, n_slots = slot_mapping.data_ptr(), k_cache.shape[0] * k_cache.shape[1]
+        kc_ptr, vc_ptr, v_ptr, v_stride = k_cache.data_ptr(), v_cache.data_ptr(), v.data_ptr(), v.stride(0)
+    check(lib.pdllm_rope_qk_store(q.data_ptr(), q.stride(0), hq, k.data_ptr(), k.stride(0), v_ptr, v_stride, hkv, d,
+                                  positions.data_ptr(), cs.data_ptr(), cs.shape[0], n, kc_ptr, vc_ptr, slots_ptr,
+                                  n_slots, _stream(q)), "rope_qk_store")

@@ -131,3 +131,25 @@ def test_product_path_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.replace("# oracle", ""), f"{f} mentions the oracle"
+
+
+def test_rotary_position_modes_follow_the_reference_formulas():
+    """fastdllm_parallelcomp.py:919-948: the three chunk modes, the two chunk-query modes and the three final
+    query modes, on values a wrong branch or a swapped argument would change."""
+    from prefilling_dllm_amd import engine_ops as eo
+    assert eo.chunk_rope_start("reuse", 7, 3, 9, 1025) == 7
+    assert eo.chunk_rope_start("continuous", 7, 3, 9, 1025) == 7 + 3 * 1025
+    assert eo.chunk_rope_start("absolute", 7, 3, 9, 1025) == 7 + 9 * 1025
+    assert eo.chunk_rope_start("continuous", 7, 3, 9, 0) == 10          # chunk_size 0 counts as 1
+    assert eo.chunk_query_rope_start("after_reused_window", 7, 100, 50, 1025) == 7 + 1025
+    assert eo.chunk_query_rope_start("after_chunk", 7, 100, 50, 1025) == 150
+    assert eo.final_query_rope_start("after_reused_window", 7, [1, 2], 8, 1025) == 7 + 1025
+    assert eo.final_query_rope_start("after_selected_chunks", 7, [1, 2], 8, 1025) == 7 + 8 * 1025
+    assert eo.final_query_rope_start("after_cache", 7, [3, 40, 12], 8, 1025) == 41
+    assert eo.final_query_rope_start("after_cache", 7, [], 8, 1025) == 7
+    for fn, args in ((eo.chunk_rope_start, ("x", 0, 0, 0, 1)), (eo.chunk_query_rope_start, ("x", 0, 0, 0, 1)),
+                     (eo.final_query_rope_start, ("x", 0, [], 0, 1))):
+        with pytest.raises(ValueError):
+            fn(*args)
+    pos = eo.chunk_positions("absolute", 2, [3, 2], [5, 1], 10)
+    assert pos.tolist() == [52, 53, 54, 12, 13]

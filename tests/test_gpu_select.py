@@ -261,3 +261,53 @@ def test_rope_matches_reference_formula(dev):
     pos = torch.randint(0, 40000, (100,), generator=gen)
     got = _ops().rope_inplace(x.clone().to(dev), pos.to(dev), cs.to(dev)).cpu()
     assert torch.equal(got, ref_ops.apply_rope(x, pos, cs))
+
+
+def test_rope_qk_store_single_launch_equals_the_three_calls(dev):
+    """pdllm_rope_qk_store = rope on q, rope on k, paged store of (rotated k, v): same bits as the three calls and
+    as the oracle; continuous chunk positions as in BASELINE config 4; slots < 0 are not stored; strided q/k/v
+    (views of a fused qkv projection)."""
+    from prefilling_dllm_amd import engine_ops as eo
+    ops = _ops()
+    gen = torch.Generator().manual_seed(15)
+    Hq, Hkv, d, P = 28, 4, 128, 256
+    lens = [300, 257, 1]
+    n = sum(lens)
+    cs = ref_ops.rope_cos_sin_cache(d, 4096, base=1000000.0)
+    qkv = torch.randn(n, (Hq + 2 * Hkv) * d, generator=gen).to(torch.bfloat16)
+    pos = eo.chunk_positions("continuous", 5, lens, [4, 0, 2], 1025)
+    assert pos[:3].tolist() == [5, 6, 7] and int(pos[300]) == 5 + 1025 and int(pos[-1]) == 5 + 2 * 1025
+    pages = torch.randperm(4, generator=gen).to(torch.int32)
+    slots = ops.slot_mapping_from_pages(pages.to(dev), n).clone()
+    slots[10:20] = -1
+
+    def views(t):
+        q = t[:, :Hq * d].view(n, Hq, d)
+        k = t[:, Hq * d:(Hq + Hkv) * d].view(n, Hkv, d)
+        v = t[:, (Hq + Hkv) * d:].view(n, Hkv, d)
+        return q, k, v
+
+    a = qkv.clone().to(dev)
+    qa, ka, va = views(a)
+    kc = torch.zeros(4, P, Hkv, d, dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    ops.rope_qk_store(qa, ka, va, pos.to(dev), cs.to(dev), kc, vc, slots)
+
+    b = qkv.clone().to(dev)
+    qb, kb, vb = views(b)
+    qb2, kb2 = qb.contiguous(), kb.contiguous()
+    ops.rope_inplace(qb2, pos.to(dev), cs.to(dev))
+    ops.rope_inplace(kb2, pos.to(dev), cs.to(dev))
+    kc2 = torch.zeros_like(kc)
+    vc2 = torch.zeros_like(kc)
+    ops.store_kvcache_unified_layout(kb2, vb.contiguous(), kc2, vc2, slots, model_type="diffusion_lm")
+    assert torch.equal(qa, qb2) and torch.equal(ka, kb2) and torch.equal(va, vb)
+    assert torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    q0, k0, _ = views(qkv)
+    assert torch.equal(qa.cpu(), ref_ops.apply_rope(q0, pos, cs))
+    assert torch.equal(ka.cpu(), ref_ops.apply_rope(k0, pos, cs))
+    # rotation only
+    c = qkv.clone().to(dev)
+    qc, kc_, _ = views(c)
+    ops.rope_qk_store(qc, kc_, None, pos.to(dev), cs.to(dev))
+    assert torch.equal(qc, qa) and torch.equal(kc_, ka)
