@@ -1258,10 +1258,10 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   const long units = (long)d->n_req * d->num_kv_heads;
   const bool fp8 = !prefill && d->k_cache != nullptr && d->max_ctx_len > 0 && d->kv_dtype == PDLLM_KV_FP8_E4M3;
   const int cus = 256;
-  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 1.5, kWide = 1.2;
+  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 1.5, kWide = 1.3;
   constexpr int kStaticLds = 66 * 1024;
   static const int js[] = {1, 2, 4, 5, 6, 8};
-  static const double upw[] = {0.25, 0.5, 1.0, 1.25, 1.5, 1.0};
+  static const double upw[] = {0.45, 0.75, 1.0, 1.25, 1.5, 1.0};
   AttnPlan best = {4, 1, (int)T, (int)T, (int)T, 1, 1, 0, 0};
   double best_cost = 1e300;
   for (int ji = 0; ji < 6; ++ji) {
