@@ -120,6 +120,32 @@ def test_config3_shape_small_batch(dev, rows):
     check(run_case(case, dev, rows_per_group=rows), oracle_case(case))
 
 
+@pytest.mark.parametrize("rows", [0, 128, 256])
+def test_ragged_requests_under_the_default_cut(dev, rows):
+    """Requests of one batch with very different numbers of selected keys (one with none at all) and the default
+    plan, whose workgroups take the first tiles of each row group side by side and then the remaining tiles:
+    a request shorter than that first part leaves the later workgroups empty pieces."""
+    case = configs.chunked_prefix_case(29, n_req=4, n_chunks=8, chunk_tokens=512, topk=6, q_len=160,
+                                       shared_prefix=False)
+    case.ranges[1] = case.ranges[1][:1]              # 512 keys
+    case.ranges[2] = []                              # only the active block
+    case.ranges[3] = [(s, l - 37) for s, l in case.ranges[3][:3]]   # ranges that end inside a page
+    ref = oracle_case(case)
+    out = run_case(case, dev, rows_per_group=rows)
+    check(out, ref)
+    # the same through the shared slot table
+    ops = _ops()
+    d = lambda t: None if t is None else t.to(dev)
+    rp, rs, rl, mr = case.range_tensors()
+    table = ops.new_slot_table(4, case.max_ctx, dev)
+    prep = ops.PreparedAttention(d(case.q), d(case.k_new), d(case.v_new), d(case.k_cache), d(case.v_cache),
+                                 d(case.block_table), d(case.q_start_loc), max_q_len=case.max_q,
+                                 max_ctx_len=case.max_ctx, ranges=(d(rp), d(rs), d(rl), mr), slot_table=table,
+                                 rows_per_group=rows)
+    prep.build_slot_table()
+    assert torch.equal(prep.run().float().cpu(), out)
+
+
 def test_context_lens_path_matches_ranges(dev):
     """The reference's decode context (first ctx_len tokens of the page table) is the single-range case."""
     case = configs.chunked_prefix_case(11, n_req=3, n_chunks=1, chunk_tokens=333, topk=1, q_len=32,
