@@ -261,6 +261,14 @@ int pdllm_topb_keep_bos(const float* scores, int64_t n_rows, int64_t chunk_len,
                         int64_t scores_stride, int64_t capacity, int32_t keep_high,
                         int32_t force_keep_first, int64_t* indices_out, pdllm_stream_t stream);
 
+/* Vote counting of the pre-eviction script (scripts/run_dream_longbench_task_fastdllm_engine_full_
+ * bridge_preevict_votetopk.sh:231-239): votes[t] += 1 for every entry t of indices [n] inside
+ * [0, length); indices outside are ignored.  votes [length] fp32 must be zeroed by the caller (counts
+ * are exact below 2^24); pdllm_topb_keep_bos over the votes of a chunk then gives the script's
+ * (-votes, index) order with the chunk's first token forced. */
+int pdllm_vote_histogram(const int64_t* indices, int64_t n, int64_t length, float* votes,
+                         pdllm_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * KV compaction / snapshot                                                   *
  * ------------------------------------------------------------------------- */

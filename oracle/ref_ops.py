@@ -428,6 +428,35 @@ def select_positions_from_token_scores(token_scores: torch.Tensor, *, capacity: 
 # logits -> confidence -> unmask (ENG:1647-1681, 2146-2157)
 # --------------------------------------------------------------------------------------
 
+def preevict_vote_topk_indices(keep_indices, full_prompt_len: int, chunk_spans, capacity: int) -> List[int]:
+    """Vote variant of the keep set, after scripts/run_dream_longbench_task_fastdllm_engine_full_bridge_
+    preevict_votetopk.sh:231-258: keep_indices[layer][head] = kept prompt positions; per chunk (start, end)
+    keep its first token and the capacity - 1 positions with the most votes, ties to the lowest index; tokens
+    between and after the chunks are all kept."""
+    votes = [0] * int(full_prompt_len)
+    for layer in keep_indices or []:
+        for head in layer or []:
+            for idx in head or []:
+                if 0 <= int(idx) < full_prompt_len:
+                    votes[int(idx)] += 1
+    keep, cursor, cap = set(), 0, int(capacity or 0)
+    for start, end in chunk_spans:
+        if start > cursor:
+            keep.update(range(cursor, start))
+        chunk_len = max(0, end - start)
+        keep_count = min(max(1, cap), chunk_len) if cap > 0 else chunk_len
+        if chunk_len > 0:
+            ranked = sorted(range(start + 1, end), key=lambda i: (-votes[i], i))
+            keep.add(start)
+            keep.update(ranked[:max(0, keep_count - 1)])
+        cursor = end
+    if cursor < full_prompt_len:
+        keep.update(range(cursor, full_prompt_len))
+    if not keep:
+        keep.update(range(full_prompt_len))
+    return sorted(keep)
+
+
 def shift_logits(logits: torch.Tensor, last_logit: Optional[torch.Tensor] = None) -> torch.Tensor:
     """ENG:1647-1656."""
     shifted = torch.empty_like(logits)

@@ -77,6 +77,7 @@ SIGNATURES = {
     "pdllm_threshold_unmask": (C.c_int, [vp, vp, vp, i64, i64, i64, f32, vp, vp, vp]),
     "pdllm_kv_copy_pages": (C.c_int, [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp]),
     "pdllm_rope_qk_store": (C.c_int, [vp, i64, i32, vp, i64, vp, i64, i32, i32, vp, vp, i64, i64, vp, vp, vp, i64, vp]),
+    "pdllm_vote_histogram": (C.c_int, [vp, i64, i64, vp, vp]),
     "pdllm_denoise_unmask": (C.c_int, [vp, i64, vp, i64, i64, i64, i64, i32, vp, i64, f32, vp, i64, vp, vp, vp, vp, vp]),
     "pdllm_chunk_select": (C.c_int, [vp, i64, vp, i64, i64, i64, i32, i64, i32, vp, i64, vp, vp, vp, vp]),
     "pdllm_rope_inplace": (C.c_int, [vp, i64, vp, vp, i64, i64, i32, i32, vp]),

@@ -256,6 +256,16 @@ __global__ __launch_bounds__(256) void evict_colsum_kernel(const float* __restri
   }
 }
 
+// votes[idx[i]] += 1 for every index inside [0, length); the counts are integers, so the order of the
+// additions does not matter
+__global__ __launch_bounds__(256) void vote_histogram_kernel(const long* __restrict__ idx, long n, long length,
+                                                             float* __restrict__ votes) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const long t = idx[i];
+  if (t >= 0 && t < length) atomicAdd(votes + t, 1.f);
+}
+
 // ---------------------------------------------------------------------------------------
 // query-to-chunk eviction scorer from q / k (bf16), fp32 math
 // ---------------------------------------------------------------------------------------
@@ -474,5 +484,16 @@ extern "C" int pdllm_token_score_pool_group(const float* scores, int64_t n_heads
   hipLaunchKernelGGL(pool_group_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)groups), dim3(256), 0,
                      static_cast<hipStream_t>(stream), scores, (long)n_heads, (long)n, pool, kernel,
                      (long)heads_per_group, out);
+  return launch_status();
+}
+
+extern "C" int pdllm_vote_histogram(const int64_t* indices, int64_t n, int64_t length, float* votes,
+                                    pdllm_stream_t stream) {
+  if (!indices || !votes) return PDLLM_ERR_NULL;
+  if (n < 0 || length <= 0 || length >= (1l << 24)) return PDLLM_ERR_SHAPE;  // counts stay exact in fp32
+  if (n == 0) return PDLLM_OK;
+  hipLaunchKernelGGL(vote_histogram_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), reinterpret_cast<const long*>(indices), (long)n, (long)length,
+                     votes);
   return launch_status();
 }

@@ -200,6 +200,46 @@ def select_positions_from_token_scores(token_scores: torch.Tensor, *, capacity: 
 # compaction / snapshot / load / chunk-local copy (ENG:525-558, 607-698)
 # ------------------------------------------------------------------------------------------
 
+def preevict_vote_topk_indices(keep_indices_per_layer_per_head: Sequence[torch.Tensor], full_prompt_len: int,
+                               chunk_spans: Sequence[Tuple[int, int]], capacity: int) -> torch.Tensor:
+    """Vote variant of the keep set (preevict_votetopk.sh:231-258): every (layer, KV head) votes for the
+    positions it kept; inside each chunk [start, end) the first token and the capacity - 1 positions with the
+    most votes (lowest index on ties) survive, tokens outside the chunks always do.  keep_indices: one int64
+    tensor [heads, keep] of prompt positions per layer (device).  Returns ascending int64 positions."""
+    n = int(full_prompt_len)
+    dev = keep_indices_per_layer_per_head[0].device if len(keep_indices_per_layer_per_head) else None
+    if n <= 0:
+        return torch.empty(0, dtype=torch.int64, device=dev)
+    if dev is None:
+        return torch.arange(n, dtype=torch.int64)
+    votes = ops.vote_histogram(torch.cat([k.reshape(-1) for k in keep_indices_per_layer_per_head]), n)
+    cap = int(capacity or 0)
+    keep = torch.zeros(n, dtype=torch.bool, device=dev)
+    cursor = 0
+    by_len: Dict[int, List[int]] = {}
+    for start, end in chunk_spans:
+        start, end = int(start), int(end)
+        if start > cursor:
+            keep[cursor:start] = True
+        if end > start:
+            by_len.setdefault(end - start, []).append(start)
+        cursor = end
+    if cursor < n:
+        keep[cursor:] = True
+    for length, starts in by_len.items():
+        if cap <= 0 or cap >= length:
+            for s0 in starts:
+                keep[s0:s0 + length] = True
+            continue
+        st = torch.as_tensor(starts, dtype=torch.int64, device=dev)
+        rows = votes[(st[:, None] + torch.arange(length, device=dev)[None, :])]       # [chunks, length]
+        sel = ops.topb_keep_bos(rows.contiguous(), max(1, cap)) + st[:, None]
+        keep[sel.reshape(-1)] = True
+    if not bool(keep.any()):
+        keep[:] = True
+    return torch.nonzero(keep).reshape(-1)
+
+
 def compact_prompt_cache_per_head(layer_cache: torch.Tensor, page_ids: torch.Tensor, keep: torch.Tensor) -> int:
     """One layer, one of K/V: token j of head h <- token keep[h][j]; gather completes before the
     write (the reference clones), so overlapping source and destination slots are safe."""

@@ -580,6 +580,17 @@ def topb_keep_bos(scores: torch.Tensor, capacity: int, keep_high: bool = True,
     return out[0] if squeeze else out
 
 
+def vote_histogram(indices: torch.Tensor, length: int) -> torch.Tensor:
+    """fp32 [length] counts of how often each position occurs in `indices` (any shape, int64); positions
+    outside [0, length) are ignored (preevict_votetopk.sh:231-239)."""
+    _need_cuda(indices)
+    idx = indices.to(torch.int64).reshape(-1).contiguous()
+    votes = torch.zeros(int(length), dtype=torch.float32, device=indices.device)
+    check(lib.pdllm_vote_histogram(idx.data_ptr(), idx.numel(), int(length), votes.data_ptr(), _stream(indices)),
+          "vote_histogram")
+    return votes
+
+
 # ----------------------------------------------------------------------------------------
 # KV gather / scatter (compaction, snapshot, load)
 # ----------------------------------------------------------------------------------------

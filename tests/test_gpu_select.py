@@ -311,3 +311,22 @@ def test_rope_qk_store_single_launch_equals_the_three_calls(dev):
     qc, kc_, _ = views(c)
     ops.rope_qk_store(qc, kc_, None, pos.to(dev), cs.to(dev))
     assert torch.equal(qc, qa) and torch.equal(kc_, ka)
+
+
+def test_vote_topk_keep_set(dev):
+    """Votes of all (layer, KV head) keep lists, then per chunk the first token + the most voted positions,
+    lowest index on ties: bit-exact with the oracle; chunks of different lengths, gaps between chunks, a
+    capacity larger than a chunk and capacity 0 (keep everything)."""
+    from prefilling_dllm_amd import engine_ops as eo
+    gen = torch.Generator().manual_seed(21)
+    n, L, H, keep = 3000, 5, 4, 600
+    spans = [(4, 1029), (1029, 2054), (2060, 2061), (2100, 2900)]
+    keep_idx = [torch.stack([torch.randperm(n + 50, generator=gen)[:keep].sort().values for _ in range(H)])
+                for _ in range(L)]
+    votes = _ops().vote_histogram(torch.cat([k.reshape(-1) for k in keep_idx]).to(dev), n).cpu()
+    want_votes = torch.bincount(torch.cat([k.reshape(-1) for k in keep_idx]).clamp(max=n), minlength=n + 1)[:n]
+    assert torch.equal(votes, want_votes.float())
+    as_lists = [[h.tolist() for h in layer] for layer in keep_idx]
+    for cap in (0, 1, 256, 900, 5000):
+        got = eo.preevict_vote_topk_indices([k.to(dev) for k in keep_idx], n, spans, cap).cpu().tolist()
+        assert got == ref_ops.preevict_vote_topk_indices(as_lists, n, spans, cap), cap

@@ -308,3 +308,31 @@ def test_fp8_page_quantisation():
     err = (deq - cache).abs()
     assert (err <= cache.abs() * 2 ** -4 + scale.view(-1, 1, 1, 1) * 2 ** -9).all()
     assert ref_ops.dequantize_pages_fp8(q, scale).dtype == torch.bfloat16
+
+
+def test_vote_topk_against_an_independent_formulation():
+    """The vote keep set (preevict_votetopk.sh:231-258) against numpy: bincount for the votes and a stable
+    argsort of the negated votes for the order, plus what the definition fixes: the first token of every chunk
+    and every token outside the chunks survive, a chunk keeps min(capacity, length) tokens, and no dropped token
+    has more votes than a kept non-first one."""
+    import numpy as np
+    rng = np.random.default_rng(3)
+    n = 90
+    spans = [(5, 30), (30, 31), (40, 80)]
+    keep_idx = [[sorted(rng.choice(n + 5, size=20, replace=False).tolist()) for _ in range(3)] for _ in range(4)]
+    votes = np.bincount(np.array([i for l in keep_idx for h in l for i in h if i < n]), minlength=n)
+    for cap in (0, 1, 4, 10, 100):
+        got = ref_ops.preevict_vote_topk_indices(keep_idx, n, spans, cap)
+        want = set(range(0, 5)) | set(range(31, 40)) | set(range(80, n))
+        for s0, e0 in spans:
+            length = e0 - s0
+            k = length if cap <= 0 else min(max(1, cap), length)
+            order = np.argsort(-votes[s0 + 1:e0], kind="stable") + s0 + 1
+            want |= {s0} | set(order[:k - 1].tolist())
+            kept = [i for i in got if s0 <= i < e0]
+            assert s0 in kept and len(kept) == k
+            dropped = [i for i in range(s0 + 1, e0) if i not in kept]
+            if dropped and len(kept) > 1:
+                assert max(votes[dropped]) <= min(votes[[i for i in kept if i != s0]])
+        assert got == sorted(want)
+    assert ref_ops.preevict_vote_topk_indices([], 4, [], 2) == [0, 1, 2, 3]
