@@ -24,6 +24,9 @@ How each function is pinned (tests/test_oracle_*.py):
   confidence / unmask : 1 / sum exp(x - max), first-max index; set formula {argmax} U {conf >= thr}
   rope : rotation preserves the norm of each (x_i, x_{i+d/2}) pair; position 0 is the identity
   fp8 : torch.float8_e4m3fn casts
+  vote keep set : numpy bincount + stable argsort, and the invariants of the definition (first token of a
+      chunk and tokens outside the chunks survive, min(capacity, length) per chunk, no dropped token
+      outvotes a kept one)
 Unpinned: nothing in this file is "parity unpinned".
 """
 from __future__ import annotations
