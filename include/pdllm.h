@@ -228,10 +228,13 @@ int pdllm_topk_lowest_index(const float* scores, int64_t n_rows, int64_t n, int6
  * heads_per_group consecutive heads summed (n_groups = n_heads / heads_per_group;
  * heads_per_group = n_heads gives the global score of
  * prefilling_dllm_eval/fastdllm_parallelcomp.py:1607-1637).  The sum runs over
- * (head, query) in index order, so it is reproducible bit for bit. */
+ * (head, query) in index order, so it is reproducible bit for bit.  workspace may be NULL; with
+ * pdllm_evict_colsum_workspace_bytes() bytes of it, few chunks are summed by one workgroup per
+ * (chunk, head, column range) in two launches (same bits, better use of the memory system). */
+int64_t pdllm_evict_colsum_workspace_bytes(int64_t n_chunks, int64_t n_heads, int64_t n_keys);
 int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t n_heads, int64_t n_queries,
-                       int64_t n_keys, int64_t heads_per_group, float* scores_out,
-                       pdllm_stream_t stream);
+                       int64_t n_keys, int64_t heads_per_group, void* workspace,
+                       int64_t workspace_bytes, float* scores_out, pdllm_stream_t stream);
 
 /* Replaces query_to_chunk_attention_scores (OPS/triton_eviction_scorer.py:114-210) and
  * the torch path of _engine_chunk_attention_head_scores (ENG:1279-1310): q [S, Hq, d],

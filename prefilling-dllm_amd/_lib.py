@@ -67,7 +67,8 @@ SIGNATURES = {
     "pdllm_vocab_workspace_bytes": (i64, [i64, i64]),
     "pdllm_chunk_score_reduce": (C.c_int, [vp, i64, i64, i32, vp, vp]),
     "pdllm_topk_lowest_index": (C.c_int, [vp, i64, i64, i64, i64, i32, vp, vp]),
-    "pdllm_evict_colsum": (C.c_int, [vp, i64, i64, i64, i64, i64, vp, vp]),
+    "pdllm_evict_colsum": (C.c_int, [vp, i64, i64, i64, i64, i64, vp, i64, vp, vp]),
+    "pdllm_evict_colsum_workspace_bytes": (i64, [i64, i64, i64]),
     "pdllm_evict_score_qk": (C.c_int, [vp, vp, i64, i64, i64, i32, i32, i32, f32, i32, i32, vp, vp, vp]),
     "pdllm_token_score_pool_group": (C.c_int, [vp, i64, i64, i32, i32, i64, vp, vp]),
     "pdllm_topb_keep_bos": (C.c_int, [vp, i64, i64, i64, i64, i32, i32, vp, vp]),

@@ -256,6 +256,67 @@ __global__ __launch_bounds__(256) void evict_colsum_kernel(const float* __restri
   }
 }
 
+// The same sums in two launches for few chunks: a workgroup owns one head and a contiguous range of
+// columns, so that every query row contributes one long contiguous segment (the narrow column blocks
+// above touch 128 bytes per row and keep few DRAM pages open); the per-head sums go to a workspace and
+// a second kernel adds the heads of a group in index order.  Same order of additions, same bits.
+constexpr int kHeadsumCols = 4;  // columns per thread at most
+__global__ __launch_bounds__(256) void evict_headsum_kernel(const float* __restrict__ probs, long n_heads, long n_q,
+                                                            long n_keys, long width, float* __restrict__ hsum) {
+  const long chunk = blockIdx.z, head = blockIdx.y;
+  const long c0 = (long)blockIdx.x * width;
+  long c1 = c0 + width;
+  c1 = c1 < n_keys ? c1 : n_keys;
+  const float* p = probs + (chunk * n_heads + head) * n_q * n_keys;
+  float acc[kHeadsumCols];
+  long col[kHeadsumCols];
+#pragma unroll
+  for (int j = 0; j < kHeadsumCols; ++j) {
+    acc[j] = 0.f;
+    const long c = c0 + threadIdx.x + 256L * j;
+    col[j] = c < c1 ? c : -1;
+  }
+  long q = 0;
+  for (; q + 8 <= n_q; q += 8) {
+    float v[8][kHeadsumCols];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int j = 0; j < kHeadsumCols; ++j) v[u][j] = col[j] >= 0 ? p[(q + u) * n_keys + col[j]] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int j = 0; j < kHeadsumCols; ++j) acc[j] += v[u][j];
+  }
+  for (; q < n_q; ++q)
+#pragma unroll
+    for (int j = 0; j < kHeadsumCols; ++j)
+      if (col[j] >= 0) acc[j] += p[q * n_keys + col[j]];
+#pragma unroll
+  for (int j = 0; j < kHeadsumCols; ++j)
+    if (col[j] >= 0) hsum[(chunk * n_heads + head) * n_keys + col[j]] = acc[j];
+}
+
+__global__ __launch_bounds__(256) void evict_groupsum_kernel(const float* __restrict__ hsum, long n_heads, long hpg,
+                                                             long n_keys, float* __restrict__ out) {
+  const long chunk = blockIdx.z, g = blockIdx.y;
+  const long c = (long)blockIdx.x * 256 + threadIdx.x;
+  if (c >= n_keys) return;
+  const long n_groups = n_heads / hpg;
+  const float* src = hsum + (chunk * n_heads + g * hpg) * n_keys + c;
+  float acc = 0.f;
+  long hh = 0;
+  for (; hh + 8 <= hpg; hh += 8) {  // eight loads in flight, added in head order
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[(hh + u) * n_keys];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += v[u];
+  }
+  for (; hh < hpg; ++hh) acc += src[hh * n_keys];
+  out[(chunk * n_groups + g) * n_keys + c] = acc;
+}
+
 // votes[idx[i]] += 1 for every index inside [0, length); the counts are integers, so the order of the
 // additions does not matter
 __global__ __launch_bounds__(256) void vote_histogram_kernel(const long* __restrict__ idx, long n, long length,
@@ -421,9 +482,15 @@ extern "C" int pdllm_topb_keep_bos(const float* scores, int64_t n_rows, int64_t 
                      force_keep_first ? 1 : 0, 0, 1, indices_out, static_cast<hipStream_t>(stream));
 }
 
+extern "C" int64_t pdllm_evict_colsum_workspace_bytes(int64_t n_chunks, int64_t n_heads, int64_t n_keys) {
+  if (n_chunks < 0 || n_heads <= 0 || n_keys <= 0) return PDLLM_ERR_SHAPE;
+  return n_chunks * n_heads * n_keys * 4;
+}
+
 extern "C" int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t n_heads,
                                   int64_t n_queries, int64_t n_keys, int64_t heads_per_group,
-                                  float* scores_out, pdllm_stream_t stream) {
+                                  void* workspace, int64_t workspace_bytes, float* scores_out,
+                                  pdllm_stream_t stream) {
   if (!probs || !scores_out) return PDLLM_ERR_NULL;
   if (n_chunks < 0 || n_heads <= 0 || n_queries <= 0 || n_keys <= 0 || heads_per_group <= 0 ||
       n_heads % heads_per_group)
@@ -433,6 +500,24 @@ extern "C" int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t 
   const size_t lds = (size_t)(n_heads * 64 * 4);
   hipStream_t st = static_cast<hipStream_t>(stream);
   const long blocks64 = (n_keys + 63) / 64 * n_chunks;
+  if (workspace != nullptr && blocks64 < 1024 && n_heads <= 65535) {
+    // few chunks: one workgroup per (chunk, head, column range), per-head sums through the workspace
+    if (workspace_bytes < n_chunks * n_heads * n_keys * 4 || ((uintptr_t)workspace % 4)) return PDLLM_ERR_WORKSPACE;
+    long parts = (512 + n_heads * n_chunks - 1) / (n_heads * n_chunks);
+    const long min_parts = (n_keys + 256 * kHeadsumCols - 1) / (256 * kHeadsumCols);
+    parts = parts < min_parts ? min_parts : parts;
+    const long width = (n_keys + parts - 1) / parts;
+    parts = (n_keys + width - 1) / width;
+    float* hsum = static_cast<float*>(workspace);
+    hipLaunchKernelGGL(evict_headsum_kernel, dim3((unsigned)parts, (unsigned)n_heads, (unsigned)n_chunks), dim3(256), 0,
+                       st, probs, (long)n_heads, (long)n_queries, (long)n_keys, width, hsum);
+    int rc = launch_status();
+    if (rc != PDLLM_OK) return rc;
+    hipLaunchKernelGGL(evict_groupsum_kernel,
+                       dim3((unsigned)((n_keys + 255) / 256), (unsigned)(n_heads / heads_per_group), (unsigned)n_chunks),
+                       dim3(256), 0, st, hsum, (long)n_heads, (long)heads_per_group, (long)n_keys, scores_out);
+    return launch_status();
+  }
   if (blocks64 >= 1024) {
     hipLaunchKernelGGL(evict_colsum_kernel<64>, dim3((unsigned)((n_keys + 63) / 64), (unsigned)n_chunks), dim3(256),
                        lds, st, probs, (long)n_heads, (long)n_queries, (long)n_keys, (long)heads_per_group, scores_out);

@@ -498,8 +498,9 @@ def evict_colsum(probs: torch.Tensor, heads_per_group: Optional[int] = None) -> 
     c, h, nq, nk = probs.shape
     hpg = h if heads_per_group is None else heads_per_group
     out = torch.empty((c, h // hpg, nk), dtype=torch.float32, device=probs.device)
-    check(lib.pdllm_evict_colsum(probs.data_ptr(), c, h, nq, nk, hpg, out.data_ptr(), _stream(probs)),
-          "evict_colsum")
+    ws = _workspace(probs.device, int(lib.pdllm_evict_colsum_workspace_bytes(c, h, nk)))
+    check(lib.pdllm_evict_colsum(probs.data_ptr(), c, h, nq, nk, hpg, _ptr(ws), 0 if ws is None else ws.numel(),
+                                 out.data_ptr(), _stream(probs)), "evict_colsum")
     return out
 
 
