@@ -311,6 +311,33 @@ def test_value_of_ones_gives_ones(dev):
     assert (out - 1.0).abs().max() <= 1e-2
 
 
+def test_limits_many_ranges_single_row_and_empty_request(dev):
+    """The edges of what a descriptor may hold: 128 ranges per request (the most the table builder accepts;
+    129 is refused), ranges of a few tokens that start and end anywhere inside pages, a request with a single
+    query row next to one with none, and a request whose ranges are empty."""
+    ops = _ops()
+    case = configs.chunked_prefix_case(37, n_req=3, n_chunks=4, chunk_tokens=512, topk=4, q_len=8,
+                                       shared_prefix=False)
+    gen = torch.Generator().manual_seed(1)
+    starts = sorted(torch.randperm(2048 - 16, generator=gen)[:128].tolist())
+    many = []
+    for i, s0 in enumerate(starts):
+        nxt = starts[i + 1] if i + 1 < len(starts) else 2048
+        many.append((s0, max(1, min(1 + i % 7, nxt - s0))))
+    case.ranges[0] = many
+    case.ranges[1] = [(5, 1)]
+    case.ranges[2] = []
+    # request 0: 8 rows, request 1: one row, request 2: no rows at all
+    case.q_start_loc = torch.tensor([0, 8, 9, 9], dtype=torch.int32)
+    case.q, case.k_new, case.v_new = case.q[:9], case.k_new[:9], case.v_new[:9]
+    ref = oracle_case(case)
+    for rows in (0, 32, 128):
+        check(run_case(case, dev, rows_per_group=rows), ref)
+    case.ranges[0] = many + [(2040, 2)]
+    with pytest.raises(NotImplementedError):
+        run_case(case, dev)
+
+
 def test_error_codes(dev):
     ops = _ops()
     q = torch.zeros(32, 4, 64, dtype=torch.bfloat16, device=dev)
