@@ -251,7 +251,9 @@ __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB
   l += psum;
 }
 
-template <int KV_FP8, int J>
+// BUF (software-pipelined variants only): the K/V copies are buffer loads with a 32-bit byte offset per
+// lane; the host selects it when every source tensor is smaller than 4 GiB.
+template <int KV_FP8, int J, bool BUF = false>
 __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_kernel(const AttnKParams p) {
   constexpr int NW = J == 8 ? 8 : 4;        // wavefronts per workgroup
   constexpr int kDmaGroups = 16 / NW;       // a tile is 16 groups of 4 rows; a wave copies this many of them
@@ -695,23 +697,31 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
       const char* vc_base = static_cast<const char*>(p.v_cache) + (long)kvh * p.cache_head_stride * 2;
       const char* kn_base = reinterpret_cast<const char*>(p.k_new + (long)q0 * p.kn_stride + kvh * kD);
       const char* vn_base = reinterpret_cast<const char*>(p.v_new + (long)q0 * p.vn_stride + kvh * kD);
+      // BUF: a buffer load with the LDS bit (resource descriptor made from the uniform base, 32-bit byte
+      // offset per lane from one 24-bit multiply-add) costs the issuing wave about 15 clk, the
+      // flat-address form 60 and more.
+      const unsigned lane_b16 = (unsigned)lane_ch << 4;
+      auto copy_row = [&](const char* base, unsigned row16, int slot, char* dst) __attribute__((always_inline)) {
+        if constexpr (BUF) {
+          const __amdgpu_buffer_rsrc_t rs =
+              __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, 0xffffffff, 0x00020000);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)dst, 16,
+                                                   __umul24((unsigned)slot, row16 << 4) + lane_b16, 0, 0, 0);
+        } else {
+          __builtin_amdgcn_global_load_lds(
+              (const __attribute__((address_space(1))) void*)(base + ((unsigned long)((unsigned)slot * row16 + lane_ch) << 4)),
+              (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+        }
+      };
       auto issue_k1 = [&](int t, int buf, int i) __attribute__((always_inline)) {
         const bool ctx = t < Tc;
-        const char* kb = ctx ? kc_base : kn_base;
-        const unsigned kr = ctx ? cache_row16 : kn_row16;
-        char* dst = lds + buf * kBufBytes + wave * 1024;
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(kb + ((unsigned long)((unsigned)nslot[i] * kr + lane_ch) << 4)),
-            (__attribute__((address_space(3))) void*)(dst + i * (NW * 1024)), 16, 0, 0);
+        copy_row(ctx ? kc_base : kn_base, ctx ? cache_row16 : kn_row16, nslot[i],
+                 lds + buf * kBufBytes + wave * 1024 + i * (NW * 1024));
       };
       auto issue_v1 = [&](int t, int buf, int i) __attribute__((always_inline)) {
         const bool ctx = t < Tc;
-        const char* vb = ctx ? vc_base : vn_base;
-        const unsigned vr = ctx ? cache_row16 : vn_row16;
-        char* dst = lds + buf * kBufBytes + kTileBytes + wave * 1024;
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(vb + ((unsigned long)((unsigned)nsv[i] * vr + lane_ch) << 4)),
-            (__attribute__((address_space(3))) void*)(dst + i * (NW * 1024)), 16, 0, 0);
+        copy_row(ctx ? vc_base : vn_base, ctx ? cache_row16 : vn_row16, nsv[i],
+                 lds + buf * kBufBytes + kTileBytes + wave * 1024 + i * (NW * 1024));
       };
       auto issue_k = [&](int t, int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -735,7 +745,7 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_k
         else if (kj == 2) lds_read_tr16_b64<base + 32 * kRowBytes>(dst, va[r][db]);
         else lds_read_tr16_b64<base + 48 * kRowBytes>(dst, va[r][db]);
       };
-      constexpr int PF = 3, NS = 16;
+      constexpr int PF = BUF ? 2 : 3, NS = 16;  // K fragments read ahead (what the register budget allows)
       auto wait_k = [&](bf16x8& x, int stp) __attribute__((always_inline)) {
         const int young = NS - 1 - stp < PF - 1 ? NS - 1 - stp : PF - 1;
         if (young == 3) lds_wait<3>(x);
@@ -1457,6 +1467,14 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
   const dim3 grid((unsigned)plan.grid), block(plan.J == 8 ? 512 : kThreads);
   const bool fp8 = has_cache && d->kv_dtype == PDLLM_KV_FP8_E4M3;
   const int dyn = dyn_lds_bytes(plan.J, d->mask_mode);
+  // 32-bit copy offsets: every tensor the copies read is smaller than 4 GiB and its rows and row
+  // indices fit the 24-bit multiply
+  const auto small = [](int64_t rows, int64_t row_bytes) {
+    return rows < (1l << 24) && row_bytes < (1l << 24) && rows * row_bytes < (1l << 32) - 4096;
+  };
+  const bool buf = !fp8 && (plan.J == 4 || plan.J == 8) && small(d->n_tokens, d->kn_stride * 2) &&
+                   small(d->n_tokens, d->vn_stride * 2) &&
+                   (!has_cache || small(d->n_pages * (int64_t)d->page_size, d->cache_token_stride * 2));
 #define PDLLM_LAUNCH(JJ)                                                                              \
   do {                                                                                                \
     if (fp8) hipLaunchKernelGGL((attn_fwd_kernel<1, JJ>), grid, block, dyn, stream, p);               \
@@ -1465,10 +1483,16 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
   switch (plan.J) {
     case 1: PDLLM_LAUNCH(1); break;
     case 2: PDLLM_LAUNCH(2); break;
-    case 4: PDLLM_LAUNCH(4); break;
+    case 4:
+      if (buf) hipLaunchKernelGGL((attn_fwd_kernel<0, 4, true>), grid, block, dyn, stream, p);
+      else PDLLM_LAUNCH(4);
+      break;
     case 5: PDLLM_LAUNCH(5); break;
     case 6: PDLLM_LAUNCH(6); break;
-    case 8: PDLLM_LAUNCH(8); break;
+    case 8:
+      if (buf) hipLaunchKernelGGL((attn_fwd_kernel<0, 8, true>), grid, block, dyn, stream, p);
+      else PDLLM_LAUNCH(8);
+      break;
     default: return PDLLM_ERR_SHAPE;
   }
 #undef PDLLM_LAUNCH

@@ -338,6 +338,33 @@ def test_limits_many_ranges_single_row_and_empty_request(dev):
         run_case(case, dev)
 
 
+def test_cache_beyond_four_gib_uses_wide_addresses(dev):
+    """The K/V copies use 32-bit byte offsets when every source tensor is below 4 GiB and 64-bit addresses
+    otherwise: the same request through a small cache and through pages at the far end of a 4.3 GB cache
+    must give the same bits."""
+    ops = _ops()
+    case = configs.chunked_prefix_case(41, n_req=2, n_chunks=6, chunk_tokens=512, topk=3, q_len=160,
+                                       shared_prefix=False)
+    ref = oracle_case(case)
+    small = run_case(case, dev)
+    check(small, ref)
+    n_small = case.k_cache.shape[0]
+    n_big = 16400                                   # x 256 tokens x 1 KiB = 4.3 GB per cache
+    shift = n_big - n_small
+    kc = torch.empty((n_big, 256, 4, 128), dtype=torch.bfloat16, device=dev)
+    vc = torch.empty_like(kc)
+    kc[shift:] = case.k_cache.to(dev)
+    vc[shift:] = case.v_cache.to(dev)
+    rp, rs, rl, mr = case.range_tensors()
+    d = lambda t: t.to(dev)
+    out = ops.sparse_decode_attention(d(case.q), d(case.k_new), d(case.v_new), kc, vc,
+                                      d(case.block_table + shift), d(case.q_start_loc), max_q_len=case.max_q,
+                                      max_ctx_len=case.max_ctx, ranges=(d(rp), d(rs), d(rl), mr))
+    torch.cuda.synchronize()
+    assert torch.equal(out.float().cpu(), small)
+    del kc, vc
+
+
 def test_error_codes(dev):
     ops = _ops()
     q = torch.zeros(32, 4, 64, dtype=torch.bfloat16, device=dev)
