@@ -745,6 +745,50 @@ def denoise_unmask(logits: torch.Tensor, block_ids: torch.Tensor, mask_token_id:
     return conf, tok, transfer.view(torch.bool), left
 
 
+class PreparedDenoiseUnmask:
+    """denoise_unmask with everything a step needs resolved once: the engine runs it after every model
+    forward on the same logits buffer and block, so outputs and workspace are allocated here and run()
+    is one library call (fastdllm_engine.py:2133-2157 without its host syncs)."""
+
+    def __init__(self, logits: torch.Tensor, block_ids: torch.Tensor, mask_token_id: int, threshold: float,
+                 shift: bool = False, last_logit: Optional[torch.Tensor] = None):
+        _need_cuda(logits, block_ids)
+        if logits.dtype != torch.bfloat16 or logits.stride(-1) != 1 or logits.dim() != 2:
+            raise ValueError("logits must be bf16 [rows, vocab]")
+        if block_ids.dtype != torch.int64 or not block_ids.is_contiguous() or block_ids.dim() != 2:
+            raise ValueError("block_ids must be contiguous int64 [n_seqs, block_len]")
+        rows, vocab = logits.shape
+        n_seqs, block_len = block_ids.shape
+        if rows != n_seqs * block_len:
+            raise ValueError("logits rows must equal n_seqs * block_len")
+        dev = logits.device
+        self.logits, self.block_ids = logits, block_ids
+        self.last_logit = None
+        ll_ptr, ll_stride = None, 0
+        if last_logit is not None:
+            self.last_logit = last_logit.to(torch.bfloat16).reshape(n_seqs, vocab).contiguous()
+            ll_ptr, ll_stride = self.last_logit.data_ptr(), self.last_logit.stride(0)
+        self.conf = torch.empty(rows, dtype=torch.float32, device=dev)
+        self.token = torch.empty(rows, dtype=torch.int64, device=dev)
+        self._transfer = torch.empty((n_seqs, block_len), dtype=torch.uint8, device=dev)
+        self.transfer = self._transfer.view(torch.bool)
+        self.left = torch.empty(n_seqs, dtype=torch.int32, device=dev)
+        need = int(lib.pdllm_vocab_workspace_bytes(rows, vocab))
+        self._ws = torch.empty(max(need, 8), dtype=torch.uint8, device=dev)
+        self._args = (logits.data_ptr(), logits.stride(0), ll_ptr, ll_stride, n_seqs, block_len, vocab,
+                      1 if shift else 0, block_ids.data_ptr(), int(mask_token_id), float(threshold),
+                      self._ws.data_ptr(), self._ws.numel(), self.conf.data_ptr(), self.token.data_ptr(),
+                      self._transfer.data_ptr(), self.left.data_ptr())
+
+    def run(self, stream: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Updates block_ids in place; returns (transfer mask, masked positions left)."""
+        st = lib.pdllm_denoise_unmask(*self._args,
+                                      torch.cuda.current_stream().cuda_stream if stream is None else stream)
+        if st != 0:
+            check(st, "PreparedDenoiseUnmask.run")
+        return self.transfer, self.left
+
+
 def rope_inplace(x: torch.Tensor, positions: torch.Tensor, cos_sin_cache: torch.Tensor) -> torch.Tensor:
     """neox rotary embedding (layers/rotary_embedding.py:6-17, 39-65) in place on bf16 x [n, heads, d]."""
     _need_cuda(x, positions, cos_sin_cache)

@@ -233,6 +233,15 @@ def test_denoise_unmask_single_call_equals_the_two_calls(dev):
         assert torch.equal(tr, tr2) and torch.equal(left, left2) and torch.equal(a_ids, b_ids)
         assert int(left[2]) == 0 and not bool(tr[2].any())
         assert int(tr[0, :7].sum()) == 0 and int(tr[0].sum()) >= 1
+        # the prepared form of the same call, run over several denoise steps until nothing is masked
+        c_ids = block.clone().to(dev)
+        prep = ops.PreparedDenoiseUnmask(logits.to(dev), c_ids, mask_id, 0.9, shift=shift, last_logit=lld)
+        tr3, left3 = prep.run()
+        assert torch.equal(tr3, tr) and torch.equal(left3, left) and torch.equal(c_ids, a_ids)
+        assert torch.equal(prep.conf, conf) and torch.equal(prep.token, tok)
+        for _ in range(L):
+            prep.run()
+        assert int(prep.left.sum()) == 0 and not bool((c_ids == mask_id).any())
 
 
 def test_argmax_first_index_on_ties(dev):
