@@ -66,7 +66,8 @@ def build_workload(torch, dev, q_len=Q_LEN, layers=LAYERS, n_req=N_REQ, seed=0):
 
 
 def algorithmic_work(q_len, ctx, n_req):
-    """Per launch (= one layer, all requests): bytes and FLOPs of SURVEY section 8(d)."""
+    """Algorithmic work of one launch (= one layer, all requests): bytes = K/V pages of the selected keys + new K/V
+    + Q read + output written; FLOPs = 4 * rows * keys * d * heads (QK^T and PV, multiply and add)."""
     by = n_req * (2 * ctx * HKV * D * 2 + 2 * q_len * HKV * D * 2 + 2 * q_len * HQ * D * 2)
     fl = n_req * 4 * q_len * (ctx + q_len) * D * HQ
     return by, fl
