@@ -254,7 +254,7 @@ __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB
 // BUF (software-pipelined variants only): the K/V copies are buffer loads with a 32-bit byte offset per
 // lane; the host selects it when every source tensor is smaller than 4 GiB.
 template <int KV_FP8, int J, bool BUF = false>
-__global__ __launch_bounds__(J == 8 ? 512 : 256, KV_FP8 ? 1 : 2) void attn_fwd_kernel(const AttnKParams p) {
+__global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void attn_fwd_kernel(const AttnKParams p) {
   constexpr int NW = J == 8 ? 8 : 4;        // wavefronts per workgroup
   constexpr int kDmaGroups = 16 / NW;       // a tile is 16 groups of 4 rows; a wave copies this many of them
   constexpr bool HAS_A = J >= 4;
@@ -1257,7 +1257,7 @@ static int dyn_lds_bytes(int J, int mask_mode) {
 // share a workgroup, which balances any shape over the CUs at the price of fp32 partials.
 // Unit of time: one wave doing one 32-row block of one 64-key tile on a CU of its own.  A
 // workgroup alone on a CU spends (fixed + blocks per wave) per tile; two workgroups sharing a CU
-// (bf16 cache, LDS footprint <= 80 KB) overlap matrix and vector work and take kPair of the
+// (at most 4 row blocks, LDS footprint <= 80 KB) overlap matrix and vector work and take kPair of the
 // serial time.  The most loaded CU sets the makespan.
 static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   const int G = d->num_q_heads / d->num_kv_heads;
@@ -1277,13 +1277,13 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   for (int ji = 0; ji < 6; ++ji) {
     const int J = js[ji];
     if (d->rows_per_group && d->rows_per_group != 32 * J) continue;
-    // 5 and 6 row blocks need more than 256 registers: fine for the fp8 path (one workgroup per CU anyway), else only on request
-    if (!d->rows_per_group && (J == 5 || J == 6) && !fp8) continue;
+    // 5 and 6 row blocks need more than 256 registers (one workgroup per CU): only on request
+    if (!d->rows_per_group && (J == 5 || J == 6)) continue;
     if (J == 8 && fp8) continue;  // the 8-wave workgroup has no room for the fp8 staging registers
     if (J == 8 && prefill && !d->rows_per_group) continue;  // coarser causal staircase: measured slower
     const long row_tiles = (nblk + J - 1) / J;
     const long cols = units * row_tiles;
-    const bool two = !fp8 && J != 8 && kStaticLds + dyn_lds_bytes(J, d->mask_mode) <= 80 * 1024;
+    const bool two = (!fp8 || J <= 4) && J != 8 && kStaticLds + dyn_lds_bytes(J, d->mask_mode) <= 80 * 1024;
     const long slots = (long)cus * (two ? 2 : 1);
     // candidate spans: whole columns, columns cut into 2..16 equal parts, and the balanced cut
     for (int cand = 0; cand <= 20; ++cand) {
