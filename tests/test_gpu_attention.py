@@ -425,3 +425,29 @@ def test_attention_layer_interface(dev):
     check(o2.view(-1, Hq, d).float().cpu(), ref2, tol=3e-2)
     # the decode step stored the new block rows behind the prompt pages
     assert torch.equal(kc[3, :block], k2.view(-1, Hkv, d))
+
+
+def test_seeded_random_shapes_and_plans(dev):
+    """40 seeded random decode cases: head layouts from MHA to 32:1 GQA, 1-9 requests, chunk lengths that are not page or
+    tile aligned, 1-200 active rows, bf16 and fp8 pages, full and causal active blocks, default and forced plans."""
+    import random
+    rnd = random.Random(20240)
+    heads = [(28, 4), (32, 32), (8, 8), (16, 2), (4, 4), (32, 1), (12, 4)]
+    for i in range(40):
+        Hq, Hkv = rnd.choice(heads)
+        n_chunks = rnd.randint(2, 10)
+        q_len = rnd.choice([1, 7, 32, 33, 64, 96, 129, 160, 200])
+        if Hq // Hkv * q_len > 2048:
+            q_len = 32
+        plan = rnd.choice([{}, {}, {}, dict(rows_per_group=rnd.choice([32, 64, 128, 256])),
+                           dict(rows_per_group=128, num_splits=rnd.randint(1, 4)),
+                           dict(rows_per_group=rnd.choice([64, 128, 256]), tiles_per_workgroup=rnd.randint(1, 9))])
+        mode = rnd.choice(["full", "full", "causal"])
+        case = configs.chunked_prefix_case(3000 + i, n_req=rnd.randint(1, 9), n_chunks=n_chunks,
+                                           chunk_tokens=rnd.choice([17, 64, 100, 255, 256, 300, 513, 640]),
+                                           topk=rnd.randint(1, n_chunks), q_len=q_len, Hq=Hq, Hkv=Hkv,
+                                           fp8=rnd.random() < 0.3, shared_prefix=rnd.random() < 0.5)
+        out = run_case(case, dev, mask_mode=mode, **plan)
+        ref = oracle_case(case, mask_mode=mode)
+        err = (out - ref).abs().max().item()
+        assert torch.isfinite(out).all() and err <= TOL_BF16, f"case {i} {case.meta} plan {plan} mask {mode}: max abs err {err}"
