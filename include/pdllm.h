@@ -214,7 +214,8 @@ int pdllm_chunk_select(const void* logits, int64_t logits_stride, const int64_t*
 /* Replaces the ranking of select_chunks_by_engine (ENG:1199-1204): per row of
  * scores [n_rows, n] (non-finite -> -inf), the k best indices by (score desc,
  * index asc), returned ascending when sorted_ascending != 0, else in rank order.
- * n <= 65536, k <= n. */
+ * n <= 65536, k <= n; rank order only for n <= 2048 (PDLLM_ERR_UNSUPPORTED beyond: the
+ * reference ranks chunks, of which there are at most a few hundred). */
 int pdllm_topk_lowest_index(const float* scores, int64_t n_rows, int64_t n, int64_t scores_stride,
                             int64_t k, int32_t sorted_ascending, int64_t* indices_out,
                             pdllm_stream_t stream);
