@@ -361,6 +361,34 @@ int pdllm_rope_qk_store(void* q, int64_t q_stride, int32_t num_q_heads, void* k,
                         int64_t n_tokens, void* k_cache, void* v_cache, const int32_t* slot_mapping,
                         int64_t n_slots, pdllm_stream_t stream);
 
+/* ------------------------------------------------------------------------- *
+ * Anchor corrections of the attention output (experimental, default off)     *
+ * ------------------------------------------------------------------------- */
+
+enum { PDLLM_ANCHOR_LEFT = 0, PDLLM_ANCHOR_RIGHT = 1, PDLLM_ANCHOR_BOTH = 2 };
+enum { PDLLM_ANCHOR_SEL_NONE = 0, PDLLM_ANCHOR_SEL_REPLACE = 1, PDLLM_ANCHOR_SEL_ADD = 2 };
+
+/* Replaces the delta / correction loops of Attention._maybe_apply_decode_delta
+ * (layers/attention/attention_v4.py:139-166) and Attention._maybe_prefill_sparse_attention
+ * (attention_v4.py:263-293).  Per sequence [q_start_loc[r], q_start_loc[r+1]) of the packed rows the
+ * anchors are the local rows anchor_offset, anchor_offset + stride, ...; anchor a spreads
+ *   delta[a] = (dense[a] - base[a]) * scale                                           (SEL_NONE)
+ *   delta[a] = (sel[a] - base[a]) * scale * valid[a]                                  (SEL_REPLACE)
+ *   delta[a] = (dense[a] - base[a]) * scale + (sel[a] - dense[a]) * sel_scale * valid[a]   (SEL_ADD)
+ * over the rows [a - left, a] (LEFT), [a, a + right] (RIGHT) or [a - left, a + right] (BOTH), clipped
+ * to the sequence, and out[r] = base[r] + sum of the deltas that reach r, anchors ascending.  Every
+ * difference, product and sum is rounded to bf16 like the reference's bf16 tensor operations.
+ * base, dense, out: bf16 [n_rows, row_elems] (row strides in elements); only the anchor rows of dense
+ * are read.  sel: bf16 [n_sel_rows, row_elems] indexed by the local anchor row (rows >= n_sel_rows read
+ * as zero and are not valid), valid[a] = sel_counts == NULL || sel_counts[a] > 0; selection modes take
+ * one sequence (n_req == 1).  out must not alias base or dense.  row_elems % 8 == 0. */
+int pdllm_anchor_delta_add(const void* base, int64_t base_stride, const void* dense, int64_t dense_stride,
+                           const void* sel, int64_t sel_stride, int64_t n_sel_rows, const int64_t* sel_counts,
+                           void* out, int64_t out_stride, const int32_t* q_start_loc, int64_t n_req,
+                           int64_t max_q_len, int64_t row_elems, int32_t stride, int32_t anchor_offset,
+                           int32_t left, int32_t right, int32_t direction, float scale, float sel_scale,
+                           int32_t sel_mode, pdllm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

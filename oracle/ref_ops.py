@@ -27,6 +27,9 @@ How each function is pinned (tests/test_oracle_*.py):
   vote keep set : numpy bincount + stable argsort, and the invariants of the definition (first token of a
       chunk and tokens outside the chunks survive, min(capacity, length) per chunk, no dropped token
       outvotes a kept one)
+  anchor corrections : hand-listed anchor / window tables for the three directions, stride 1 with a zero window
+      reproduces the dense result, an unchanged prompt gives a zero delta, the selection modes reduce to the plain
+      mode for selection == dense
 Unpinned: nothing in this file is "parity unpinned".
 """
 from __future__ import annotations
@@ -240,6 +243,115 @@ def chunk_prefill_attention(q, k, v, cu_seqlens, *, causal=True, sm_scale=None, 
     cu = [int(x) for x in cu_seqlens]
     return sparse_decode_attention(q, k, v, None, None, None, cu, None,
                                    mask_mode="causal" if causal else "full", sm_scale=sm_scale, dtype=dtype)
+
+
+# --------------------------------------------------------------------------------------
+# experimental anchor corrections (ATT:86-293, default off)
+# --------------------------------------------------------------------------------------
+
+def anchor_windows(seq_len: int, state: dict):
+    """Anchors and the rows each one corrects: ATT:113-125 (defaults and clamps) and ATT:151-165 (windows)."""
+    stride = max(1, int(state.get("stride", 4)))
+    left = max(0, int(state.get("left", stride - 1)))
+    right = max(0, int(state.get("right", 0)))
+    direction = (state.get("direction") or "left").lower()
+    anchor_offset = int(state.get("anchor_offset", stride - 1))
+    if anchor_offset < 0:
+        anchor_offset = stride - 1
+    anchor_offset = min(anchor_offset, stride - 1)
+    anchors = list(range(anchor_offset, seq_len, stride))
+    windows = []
+    for anchor in anchors:
+        if direction == "right":
+            rows = range(anchor, min(seq_len - 1, anchor + right) + 1)
+        elif direction == "both":
+            rows = range(max(0, anchor - left), min(seq_len - 1, anchor + right) + 1)
+        else:
+            rows = range(max(0, anchor - left), anchor + 1)
+        windows.append(list(rows))
+    return anchors, windows
+
+
+def anchor_delta_add(base, delta, windows):
+    """ATT:150-166: correction = zeros_like(base); correction[rows] += delta[idx] per anchor, ascending; base +
+    correction.  base [S, H, d], delta [A, H, d]; computed in the dtype of the tensors (bf16 tensors round after every
+    operation, as the reference's do)."""
+    correction = torch.zeros_like(base)
+    for idx, rows in enumerate(windows):
+        if rows:
+            correction[rows] += delta[idx:idx + 1]
+    return base + correction
+
+
+def decode_delta(o, q, k_new, v_new, full_k, full_v, state, *, active_mask=None, sm_scale=None):
+    """Attention._maybe_apply_decode_delta (ATT:86-166): the anchor rows attend to [full prompt || active rows]
+    (prompt keys all visible, active keys by active_mask[anchors] or all), delta = (dense - o[anchors]) * scale is
+    spread over each anchor's window.  o / q [S, Hq, d], k_new / v_new [S, Hkv, d], full_k / full_v [P, Hkv, d].
+    Arithmetic in the dtype of o."""
+    S, _, d = q.shape
+    anchors, windows = anchor_windows(S, state)
+    if not anchors:
+        return o
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(d)
+    k_all = torch.cat([full_k.to(k_new.dtype), k_new], dim=0)
+    v_all = torch.cat([full_v.to(v_new.dtype), v_new], dim=0)
+    am = torch.ones((len(anchors), S), dtype=torch.bool) if active_mask is None else active_mask[anchors].to(torch.bool)
+    mask = torch.cat([torch.ones((len(anchors), full_k.shape[0]), dtype=torch.bool), am], dim=1)
+    dense_anchor = _sdpa(q[anchors], k_all, v_all, mask, sm_scale, torch.float32).to(o.dtype)
+    delta = (dense_anchor - o[anchors]) * float(state.get("scale", 1.0))
+    return anchor_delta_add(o, delta, windows)
+
+
+def prefill_sparse_attention(q, k, v, base_mask, keep, state, *, sm_scale=None, selection_outputs=None,
+                             selection_counts=None, out_dtype=torch.float32):
+    """Attention._maybe_prefill_sparse_attention (ATT:168-293) for one layer: keys outside `keep` (and before
+    full_prompt_len) are masked on top of base_mask; with a delta mode the anchor rows are corrected towards the
+    dense result (or the stored selection outputs).  q [S, Hq, d], k / v [S, Hkv, d], base_mask [S, S] bool.
+    The attention is computed in fp32 and cast to out_dtype, the correction runs in out_dtype."""
+    S, Hq, d = q.shape
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(d)
+    key_mask = torch.zeros(S, dtype=torch.bool)
+    valid_keep = keep.reshape(-1).long()
+    valid_keep = valid_keep[(valid_keep >= 0) & (valid_keep < S)]
+    key_mask[valid_keep] = True
+    full_prompt_len = int(state.get("full_prompt_len", S))
+    if 0 <= full_prompt_len < S:
+        key_mask[full_prompt_len:] = True
+    base_mask = base_mask.to(torch.bool)
+    o_sparse = _sdpa(q, k, v, base_mask & key_mask.unsqueeze(0), sm_scale, torch.float32).to(out_dtype)
+    delta_mode = (state.get("delta_mode") or "none").lower()
+    if delta_mode in {"none", "off", "0", ""}:
+        return o_sparse
+    anchors, windows = anchor_windows(S, state)
+    if not anchors:
+        return o_sparse
+    sparse_anchor = o_sparse[anchors]
+    selection_mode = (state.get("selection_mode") or "none").lower()
+    selection_anchor = selection_valid = None
+    if selection_mode in {"selection_dense_replace", "selection_dense_add"} and selection_outputs is not None \
+            and selection_outputs.shape[0] > 0 and selection_outputs.shape[1] == Hq:
+        at = torch.tensor(anchors)
+        in_range = at < selection_outputs.shape[0]
+        safe = at.clamp_max(selection_outputs.shape[0] - 1)
+        selection_anchor = torch.zeros_like(sparse_anchor)
+        selection_anchor[in_range] = selection_outputs.to(out_dtype)[safe][in_range]
+        selection_valid = ((selection_counts[safe] > 0) & in_range) if selection_counts is not None else in_range
+    dense_anchor = None
+    if selection_mode != "selection_dense_replace":
+        dense_anchor = _sdpa(q[anchors], k, v, base_mask[anchors], sm_scale, torch.float32).to(out_dtype)
+    if selection_mode == "selection_dense_replace":
+        if selection_anchor is None or not bool(selection_valid.any()):
+            return o_sparse
+        delta = (selection_anchor - sparse_anchor) * float(state.get("scale", 1.0))
+        delta = delta * selection_valid.view(-1, 1, 1).to(delta.dtype)
+    else:
+        delta = (dense_anchor - sparse_anchor) * float(state.get("scale", 1.0))
+        if selection_mode == "selection_dense_add" and selection_anchor is not None:
+            sd = (selection_anchor - dense_anchor) * float(state.get("selection_scale", 1.0))
+            delta = delta + sd * selection_valid.view(-1, 1, 1).to(sd.dtype)
+    return anchor_delta_add(o_sparse, delta, windows)
 
 
 def split_token_chunks(token_ids: Sequence[int], chunk_size: int, split_from_tail: bool = False):

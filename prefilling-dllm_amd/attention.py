@@ -8,8 +8,10 @@ paged cache through the slot mapping, and attends
   * decode: the active rows to [visible prefix pages || active rows] without the dense
     load_kvcache staging copy -- attention_v4.py:368-397.
 
-The experimental decode-delta / sparse-prefill corrections of the reference (default off) are not
-part of this layer."""
+The experimental corrections of the reference (default off) are here too: the decode delta
+(attention_v4.py:86-166: anchors re-attend to the full prompt, the difference is spread over their
+neighbours) and the sparse prefill with its anchor delta (attention_v4.py:168-293).  The denser
+attention is computed for every row and read at the anchors."""
 from __future__ import annotations
 
 import os
@@ -53,7 +55,10 @@ class Attention(nn.Module):
         if context.block_mask is not None:
             mask_mode, dense = "dense", context.block_mask
         if context.is_prefill:
-            if mask_mode == "dense":
+            o = self._maybe_prefill_sparse_attention(q, k, v, context)
+            if o is not None:
+                pass
+            elif mask_mode == "dense":
                 o = ops.sparse_decode_attention(q, k, v, None, None, None, context.cu_seqlens_q,
                                                 max_q_len=int(context.max_seqlen_q), max_ctx_len=0,
                                                 mask_mode="dense", mask=dense, sm_scale=self.scale)
@@ -67,4 +72,146 @@ class Attention(nn.Module):
                                             max_q_len=int(context.max_seqlen_q), max_ctx_len=max_ctx if has_cache else 0,
                                             context_lens=context.context_lens, ranges=context.ranges,
                                             mask_mode=mask_mode, mask=dense, sm_scale=self.scale)
+            o = self._maybe_apply_decode_delta(o, q, k, v, context)
         return o.view(-1, self.num_heads * self.head_dim)
+
+    # ---- experimental corrections (default off) ----
+
+    @staticmethod
+    def _debug_stats(state, delta_abs_max: float, n_anchors: int) -> None:
+        state["calls"] = int(state.get("calls", 0)) + 1
+        state["nonzero_calls"] = int(state.get("nonzero_calls", 0)) + int(delta_abs_max > 0.0)
+        state["max_abs"] = max(float(state.get("max_abs", 0.0)), delta_abs_max)
+        state["anchor_count"] = int(state.get("anchor_count", 0)) + n_anchors
+
+    def _maybe_apply_decode_delta(self, o, q, k_new, v_new, context):
+        """attention_v4.py:86-166.  The packed active rows are one sequence, as in the reference."""
+        state = getattr(context, "decode_delta_state", None)
+        if not state or not state.get("enabled", False) or self.layer_idx < 0:
+            return o
+        full_k_by_layer, full_v_by_layer = state.get("full_k"), state.get("full_v")
+        if full_k_by_layer is None or full_v_by_layer is None or self.layer_idx >= len(full_k_by_layer):
+            return o
+        full_k, full_v = full_k_by_layer[self.layer_idx], full_v_by_layer[self.layer_idx]
+        if full_k is None or full_v is None or full_k.numel() == 0:
+            return o
+        seq_len = q.shape[0]
+        ap = ops.anchor_params(state, seq_len)
+        if ap is None:
+            return o
+        stride, offset, left, right, direction = ap
+        # the full prompt K/V [S, Hkv, d] as pages of a cache of its own (one copy, where the reference concatenates)
+        n_prompt, page = int(full_k.shape[0]), 256
+        pages = (n_prompt + page - 1) // page
+        kc = torch.empty((pages, page, self.num_kv_heads, self.head_dim), dtype=k_new.dtype, device=k_new.device)
+        vc = torch.empty_like(kc)
+        kc.view(-1, self.num_kv_heads, self.head_dim)[:n_prompt].copy_(full_k)
+        vc.view(-1, self.num_kv_heads, self.head_dim)[:n_prompt].copy_(full_v)
+        dev = q.device
+        one_seq = torch.tensor([0, seq_len], dtype=torch.int32, device=dev)
+        mask_mode = "dense" if context.block_mask is not None else context.mask_kind
+        dense = ops.sparse_decode_attention(q, k_new, v_new, kc, vc,
+                                            torch.arange(pages, dtype=torch.int32, device=dev).view(1, -1), one_seq,
+                                            max_q_len=seq_len, max_ctx_len=n_prompt,
+                                            context_lens=torch.tensor([n_prompt], dtype=torch.int32, device=dev),
+                                            mask_mode=mask_mode, mask=context.block_mask, sm_scale=self.scale)
+        scale = float(state.get("scale", 1.0))
+        if state.get("debug", False):
+            anchors = torch.arange(offset, seq_len, stride, device=dev)
+            delta = (dense.index_select(0, anchors) - o.index_select(0, anchors)) * scale
+            self._debug_stats(state, float(delta.abs().max().item()) if delta.numel() else 0.0, int(anchors.numel()))
+        return ops.anchor_delta_add(o, dense, one_seq, max_q_len=seq_len, stride=stride, anchor_offset=offset,
+                                    left=left, right=right, direction=direction, scale=scale)
+
+    def _maybe_prefill_sparse_attention(self, q, k, v, context):
+        """attention_v4.py:168-293.  None = not active, the caller runs the ordinary prefill."""
+        state = getattr(context, "prefill_sparse_state", None)
+        if not state or not state.get("enabled", False):
+            return None
+        if self.model_type != "diffusion_lm" or self.layer_idx < 0:
+            return None
+        keep_by_layer = state.get("keep_indices")
+        if keep_by_layer is None or self.layer_idx >= len(keep_by_layer):
+            return None
+        base_mask = context.block_mask
+        if base_mask is None:
+            return None
+        seq_len, dev = q.shape[0], q.device
+        layer_keep = keep_by_layer[self.layer_idx]
+        if layer_keep is None or layer_keep.numel() == 0:
+            return None
+        valid_keep = layer_keep.to(device=dev, dtype=torch.long).reshape(-1)
+        valid_keep = valid_keep[(valid_keep >= 0) & (valid_keep < seq_len)]
+        if valid_keep.numel() == 0:
+            return None
+        key_mask = torch.zeros(seq_len, dtype=torch.bool, device=dev)
+        key_mask[valid_keep] = True
+        full_prompt_len = int(state.get("full_prompt_len", seq_len))
+        if 0 <= full_prompt_len < seq_len:
+            key_mask[full_prompt_len:] = True
+        if state.get("debug", False):
+            active_keys = int(key_mask.sum().item())
+            state["union_min"] = min(int(state.get("union_min", active_keys)), active_keys)
+            state["union_max"] = max(int(state.get("union_max", active_keys)), active_keys)
+        base_mask = base_mask.to(device=dev, dtype=torch.bool)
+        one_seq = torch.tensor([0, seq_len], dtype=torch.int32, device=dev)
+
+        def attend(mask):
+            return ops.sparse_decode_attention(q, k, v, None, None, None, one_seq, max_q_len=seq_len, max_ctx_len=0,
+                                               mask_mode="dense", mask=mask, sm_scale=self.scale)
+
+        o_sparse = attend(base_mask & key_mask.unsqueeze(0))
+        delta_mode = (state.get("delta_mode") or "none").lower()
+        if delta_mode in {"none", "off", "0", ""}:
+            return o_sparse
+        if delta_mode not in {"s4_left3", "delta_s4_left3", "sampled_delta_s4_left3"}:
+            raise ValueError(f"Unsupported prefill_delta_mode: {delta_mode}")
+        ap = ops.anchor_params(state, seq_len)
+        if ap is None:
+            return o_sparse
+        stride, offset, left, right, direction = ap
+
+        selection_mode = (state.get("selection_mode") or "none").lower()
+        selection_dense = state.get("selection_dense")
+        sel = counts = None
+        if selection_mode in {"selection_dense_replace", "selection_dense_add"} and selection_dense:
+            outputs_by_layer = selection_dense.get("outputs") if isinstance(selection_dense, dict) else None
+            counts_by_layer = selection_dense.get("counts") if isinstance(selection_dense, dict) else None
+            if outputs_by_layer is not None and self.layer_idx < len(outputs_by_layer):
+                layer_outputs = outputs_by_layer[self.layer_idx]
+                if layer_outputs is not None and layer_outputs.shape[0] > 0 and layer_outputs.shape[1] == self.num_heads:
+                    sel = layer_outputs.to(device=dev, dtype=o_sparse.dtype).contiguous()
+                    if counts_by_layer is not None and self.layer_idx < len(counts_by_layer) and \
+                            counts_by_layer[self.layer_idx] is not None:
+                        counts = counts_by_layer[self.layer_idx].to(dev)
+        scale = float(state.get("scale", 1.0))
+        kw = dict(max_q_len=seq_len, stride=stride, anchor_offset=offset, left=left, right=right, direction=direction,
+                  scale=scale)
+        anchors = torch.arange(offset, seq_len, stride, device=dev)
+
+        def any_valid():
+            in_range = anchors < sel.shape[0]
+            if counts is None:
+                return bool(in_range.any().item())
+            safe = anchors.clamp_max(sel.shape[0] - 1)
+            return bool(((counts.index_select(0, safe) > 0) & in_range).any().item())
+
+        if selection_mode == "selection_dense_replace":
+            if sel is None or not any_valid():
+                return o_sparse
+            out = ops.anchor_delta_add(o_sparse, None, one_seq, sel=sel, sel_counts=counts, sel_mode="replace", **kw)
+            state["selection_used_calls"] = int(state.get("selection_used_calls", 0)) + 1
+            dense = None
+        else:
+            dense = attend(base_mask)
+            if selection_mode == "selection_dense_add" and sel is not None:
+                out = ops.anchor_delta_add(o_sparse, dense, one_seq, sel=sel, sel_counts=counts, sel_mode="add",
+                                           sel_scale=float(state.get("selection_scale", 1.0)), **kw)
+                state["selection_used_calls"] = int(state.get("selection_used_calls", 0)) + 1
+            else:
+                out = ops.anchor_delta_add(o_sparse, dense, one_seq, **kw)
+        if state.get("debug", False):
+            # largest |out - o_sparse| over the anchor rows stands in for the reference's max |delta|
+            diff = (out.index_select(0, anchors).float() - o_sparse.index_select(0, anchors).float()).abs()
+            self._debug_stats(state, float(diff.max().item()) if diff.numel() else 0.0, int(anchors.numel()))
+        return out

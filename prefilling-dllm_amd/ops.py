@@ -831,3 +831,64 @@ def rope_qk_store(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], p
     check(lib.pdllm_rope_qk_store(q.data_ptr(), q.stride(0), hq, k.data_ptr(), k.stride(0), v_ptr, v_stride, hkv, d,
                                   positions.data_ptr(), cs.data_ptr(), cs.shape[0], n, kc_ptr, vc_ptr, slots_ptr,
                                   n_slots, _stream(q)), "rope_qk_store")
+
+
+# ----------------------------------------------------------------------------------------------
+# anchor corrections of the attention output
+# ----------------------------------------------------------------------------------------------
+
+def anchor_params(state: dict, seq_len: int) -> Optional[Tuple[int, int, int, int, int]]:
+    """(stride, anchor_offset, left, right, direction) from a decode-delta / sparse-prefill state dict with the
+    reference's defaults and clamps (attention_v4.py:113-125, 226-236), or None when the sequence has no anchor.
+    direction: 0 left, 1 right, 2 both."""
+    stride = max(1, int(state.get("stride", 4)))
+    left = max(0, int(state.get("left", stride - 1)))
+    right = max(0, int(state.get("right", 0)))
+    direction = {"right": 1, "both": 2}.get((state.get("direction") or "left").lower(), 0)
+    anchor_offset = int(state.get("anchor_offset", stride - 1))
+    if anchor_offset < 0:
+        anchor_offset = stride - 1
+    anchor_offset = min(anchor_offset, stride - 1)
+    if seq_len <= anchor_offset:
+        return None
+    return stride, anchor_offset, left, right, direction
+
+
+def anchor_delta_add(base: torch.Tensor, dense: Optional[torch.Tensor], q_start_loc: torch.Tensor, *, max_q_len: int,
+                     stride: int, anchor_offset: int, left: int, right: int, direction: int, scale: float = 1.0,
+                     sel: Optional[torch.Tensor] = None, sel_counts: Optional[torch.Tensor] = None,
+                     sel_scale: float = 1.0, sel_mode: str = "none") -> torch.Tensor:
+    """base + the window sums of the anchor deltas (attention_v4.py:139-166, 263-293), rounded to bf16 where the
+    reference's bf16 tensor operations round.  base / dense [n_rows, heads, d] bf16 (dense is read at the anchor rows
+    only); sel [n_sel_rows, heads, d] bf16 with sel_mode "replace" / "add".  Returns a new tensor."""
+    _need_cuda(base, q_start_loc)
+    mode = {"none": 0, "replace": 1, "add": 2}[sel_mode]
+    rows = base.shape[0]
+    row_elems = base.numel() // max(rows, 1)
+    b2 = base.reshape(rows, row_elems)
+    if b2.dtype != torch.bfloat16 or b2.stride(-1) != 1:
+        raise ValueError("base must be bf16 with contiguous rows")
+    out = torch.empty_like(b2)
+
+    def rows_of(t, name):
+        if t is None:
+            return None, 0, 0
+        t2 = t.reshape(t.shape[0], row_elems)
+        if t2.dtype != torch.bfloat16 or t2.stride(-1) != 1:
+            raise ValueError(f"{name} must be bf16 with contiguous rows of {row_elems} elements")
+        return t2, t2.stride(0), t2.shape[0]
+
+    d2, d_stride, d_rows = rows_of(dense, "dense")
+    if d2 is not None and d_rows != rows:
+        raise ValueError("dense must have one row per base row")
+    s2, s_stride, s_rows = rows_of(sel, "sel")
+    cnt = None if sel_counts is None else sel_counts.to(device=base.device, dtype=torch.int64).contiguous()
+    if cnt is not None and cnt.numel() < s_rows:
+        raise ValueError("sel_counts must have one entry per selection row")
+    qsl = q_start_loc.to(torch.int32).contiguous()
+    check(lib.pdllm_anchor_delta_add(b2.data_ptr(), b2.stride(0), _ptr(d2), d_stride, _ptr(s2), s_stride, s_rows,
+                                     _ptr(cnt), out.data_ptr(), out.stride(0), qsl.data_ptr(), qsl.numel() - 1,
+                                     int(max_q_len), row_elems, int(stride), int(anchor_offset), int(left), int(right),
+                                     int(direction), float(scale), float(sel_scale), mode, _stream(base)),
+          "anchor_delta_add")
+    return out.view(base.shape)

@@ -336,3 +336,95 @@ def test_vote_topk_against_an_independent_formulation():
                 assert max(votes[dropped]) <= min(votes[[i for i in kept if i != s0]])
         assert got == sorted(want)
     assert ref_ops.preevict_vote_topk_indices([], 4, [], 2) == [0, 1, 2, 3]
+
+
+# ---- experimental anchor corrections ----
+
+def test_anchor_windows_hand_listed_tables():
+    """Anchors and windows read off the reference loops by hand (ATT:113-125, 151-165)."""
+    aw = ref_ops.anchor_windows
+    assert aw(10, {}) == ([3, 7], [[0, 1, 2, 3], [4, 5, 6, 7]])                     # stride 4, left 3, offset 3
+    assert aw(10, dict(direction="right", right=2)) == ([3, 7], [[3, 4, 5], [7, 8, 9]])
+    assert aw(9, dict(direction="right", right=3)) == ([3, 7], [[3, 4, 5, 6], [7, 8]])   # clipped at the end
+    assert aw(10, dict(direction="both", left=1, right=1)) == ([3, 7], [[2, 3, 4], [6, 7, 8]])
+    assert aw(9, dict(anchor_offset=0)) == ([0, 4, 8], [[0], [1, 2, 3, 4], [5, 6, 7, 8]])
+    assert aw(10, dict(anchor_offset=-5))[0] == [3, 7]                              # negative -> stride - 1
+    assert aw(10, dict(anchor_offset=99))[0] == [3, 7]                              # clamped to stride - 1
+    assert aw(10, dict(stride=2, left=5))[1][1] == [0, 1, 2, 3]                      # overlapping windows
+    assert aw(3, {}) == ([], [])
+    assert aw(7, dict(stride=0, left=0))[0] == list(range(7))                       # stride < 1 -> 1
+
+
+def test_decode_delta_reduces_to_known_cases():
+    gen = torch.Generator().manual_seed(5)
+    Hq, Hkv, d, S, P = 8, 2, 32, 12, 40
+    q = torch.randn(S, Hq, d, generator=gen)
+    k, v = torch.randn(S, Hkv, d, generator=gen), torch.randn(S, Hkv, d, generator=gen)
+    fk, fv = torch.randn(P, Hkv, d, generator=gen), torch.randn(P, Hkv, d, generator=gen)
+    keep = torch.arange(0, P, 3)                                                    # the sparse prefix: every third key
+    full = torch.ones(S, S + keep.numel(), dtype=torch.bool)
+    o = ref_ops._sdpa(q, torch.cat([fk[keep], k]), torch.cat([fv[keep], v]), full, d ** -0.5)
+    dense_all = ref_ops._sdpa(q, torch.cat([fk, k]), torch.cat([fv, v]), torch.ones(S, S + P, dtype=torch.bool), d ** -0.5)
+    # every row an anchor with a window of one row and scale 1: the result is the dense attention itself
+    got = ref_ops.decode_delta(o, q, k, v, fk, fv, dict(stride=1, left=0))
+    assert (got - dense_all).abs().max() < 1e-5
+    # scale 0.5 moves every row half way
+    got = ref_ops.decode_delta(o, q, k, v, fk, fv, dict(stride=1, left=0, scale=0.5))
+    assert (got - (o + dense_all) / 2).abs().max() < 1e-5
+    # a "full" prompt equal to the sparse prefix changes nothing
+    got = ref_ops.decode_delta(o, q, k, v, fk[keep], fv[keep], {})
+    assert (got - o).abs().max() < 1e-5
+    # default windows: rows 0-3 receive the delta of row 3, rows 4-7 that of row 7, rows 8-11 that of row 11
+    got = ref_ops.decode_delta(o, q, k, v, fk, fv, {})
+    for r in range(S):
+        a = r // 4 * 4 + 3
+        assert (got[r] - (o[r] + dense_all[a] - o[a])).abs().max() < 1e-5
+    # an active mask only changes the anchors' view of the active keys
+    am = torch.tril(torch.ones(S, S, dtype=torch.bool))
+    got = ref_ops.decode_delta(o, q, k, v, fk, fv, dict(stride=1, left=0), active_mask=am)
+    causal = ref_ops._sdpa(q, torch.cat([fk, k]), torch.cat([fv, v]),
+                           torch.cat([torch.ones(S, P, dtype=torch.bool), am], 1), d ** -0.5)
+    assert (got - causal).abs().max() < 1e-5
+
+
+def test_prefill_sparse_reduces_to_known_cases():
+    gen = torch.Generator().manual_seed(6)
+    Hq, Hkv, d, S = 4, 2, 32, 14
+    q = torch.randn(S, Hq, d, generator=gen)
+    k, v = torch.randn(S, Hkv, d, generator=gen), torch.randn(S, Hkv, d, generator=gen)
+    causal = torch.tril(torch.ones(S, S, dtype=torch.bool))
+    dense = ref_ops._sdpa(q, k, v, causal, d ** -0.5)
+    every = torch.arange(S)
+    # all keys kept: the sparse prefill is the dense one, with or without the delta
+    for st in ({}, dict(delta_mode="s4_left3")):
+        assert (ref_ops.prefill_sparse_attention(q, k, v, causal, every, st) - dense).abs().max() < 1e-6
+    # a subset: the same as attention over the gathered keys with the causal mask gathered alike
+    keep = torch.tensor([0, 2, 3, 7, 8, 12, 40, -1])                                 # out-of-range entries are ignored
+    kk = keep[(keep >= 0) & (keep < S)]
+    sub = ref_ops._sdpa(q, k[kk], v[kk], causal[:, kk], d ** -0.5)
+    got = ref_ops.prefill_sparse_attention(q, k, v, causal, keep, {})
+    assert (got - sub).abs().max() < 1e-6
+    # keys from full_prompt_len on are always visible
+    got = ref_ops.prefill_sparse_attention(q, k, v, causal, keep, dict(full_prompt_len=10))
+    kk2 = torch.tensor([0, 2, 3, 7, 8, 10, 11, 12, 13])
+    assert (got - ref_ops._sdpa(q, k[kk2], v[kk2], causal[:, kk2], d ** -0.5)).abs().max() < 1e-6
+    # delta: anchors 3, 7, 11 land on the dense result, their windows move by the same amount; rows 12, 13 stay
+    got = ref_ops.prefill_sparse_attention(q, k, v, causal, keep, dict(delta_mode="s4_left3"))
+    for r in range(S):
+        a = r // 4 * 4 + 3
+        want = sub[r] + (dense[a] - sub[a]) if a < S else sub[r]
+        assert (got[r] - want).abs().max() < 1e-5
+    with_sel = dict(delta_mode="s4_left3", selection_mode="selection_dense_add", selection_scale=0.7)
+    # selection outputs equal to the dense result: both selection modes give the plain correction
+    g_add = ref_ops.prefill_sparse_attention(q, k, v, causal, keep, with_sel, selection_outputs=dense)
+    assert (g_add - got).abs().max() < 1e-5
+    rep = dict(delta_mode="s4_left3", selection_mode="selection_dense_replace")
+    g_rep = ref_ops.prefill_sparse_attention(q, k, v, causal, keep, rep, selection_outputs=dense)
+    assert (g_rep - got).abs().max() < 1e-5
+    # replace with counts == 0 everywhere, or no selection at all: the sparse result is returned
+    g0 = ref_ops.prefill_sparse_attention(q, k, v, causal, keep, rep, selection_outputs=dense,
+                                          selection_counts=torch.zeros(S, dtype=torch.long))
+    assert torch.equal(g0, sub.to(g0.dtype)) or (g0 - sub).abs().max() < 1e-6
+    # a selection shorter than the sequence: anchors past its end are not valid (replace: no correction there)
+    g_short = ref_ops.prefill_sparse_attention(q, k, v, causal, keep, rep, selection_outputs=dense[:8])
+    assert (g_short[:8] - got[:8]).abs().max() < 1e-5 and (g_short[8:] - sub[8:]).abs().max() < 1e-6
