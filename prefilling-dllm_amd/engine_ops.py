@@ -148,6 +148,21 @@ class PrefixPageAllocator:
 # chunk ranking (ENG:1199-1204)
 # ------------------------------------------------------------------------------------------
 
+def split_token_chunks(token_ids: Sequence[int], chunk_size: int, split_from_tail: bool = False) -> List[List[int]]:
+    """Prompt -> consecutive chunks of chunk_size tokens (prefilling_dllm_eval/fastdllm_parallelcomp.py:158-180).
+    The short chunk is the last one, or the first one with split_from_tail; a non-positive chunk_size or a prompt
+    that fits gives one chunk, an empty prompt none."""
+    ids = list(token_ids)
+    n = len(ids)
+    if n == 0:
+        return []
+    if chunk_size <= 0 or n <= chunk_size:
+        return [ids]
+    first = n % chunk_size if split_from_tail else 0
+    cuts = ([0] if first else []) + list(range(first, n, chunk_size)) + [n]
+    return [ids[a:b] for a, b in zip(cuts[:-1], cuts[1:])]
+
+
 def select_chunks_from_scores(scores: torch.Tensor, topk_chunks: int, keep_first_chunk: bool = False) -> torch.Tensor:
     """Ranking tail of select_chunks_by_engine: non-finite -> -inf, stable descending order
     (lowest index first on ties), the top `topk_chunks` of the non-forced chunks plus chunk 0 when

@@ -153,3 +153,19 @@ def test_rotary_position_modes_follow_the_reference_formulas():
             fn(*args)
     pos = eo.chunk_positions("absolute", 2, [3, 2], [5, 1], 10)
     assert pos.tolist() == [52, 53, 54, 12, 13]
+
+
+def test_split_token_chunks_cases():
+    """Chunking of the prompt (fastdllm_parallelcomp.py:158-180): hand-listed cases and the oracle on a sweep."""
+    from oracle import ref_ops
+    from prefilling_dllm_amd import engine_ops
+    f = engine_ops.split_token_chunks
+    assert f([], 4) == []
+    assert f([1, 2, 3], 4) == [[1, 2, 3]] and f([1, 2, 3], 0) == [[1, 2, 3]] and f([1, 2, 3], -2) == [[1, 2, 3]]
+    assert f(range(10), 4) == [[0, 1, 2, 3], [4, 5, 6, 7], [8, 9]]
+    assert f(range(10), 4, split_from_tail=True) == [[0, 1], [2, 3, 4, 5], [6, 7, 8, 9]]
+    assert f(range(8), 4, split_from_tail=True) == [[0, 1, 2, 3], [4, 5, 6, 7]]
+    for n in range(0, 40):
+        for c in (1, 2, 3, 7, 16):
+            for tail in (False, True):
+                assert f(range(n), c, tail) == ref_ops.split_token_chunks(range(n), c, tail)
