@@ -1136,26 +1136,32 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const MergeParams m) {
   const int np = (m.head > 0 ? 1 : 0) + (tail_at + tail_len - 1) / m.span - tail_at / m.span + 1;
   if (np == 1) return;
   const long R = ((long)(q0 + tq) * m.Hq + head) * m.max_pieces;
-  float M = -INFINITY;
-  for (int s = 0; s < np; ++s) M = fmaxf(M, m.ws_lse[R + s]);
+  // Four pieces at a time: their log-sum-exps and partial rows are fetched together (one round trip), then
+  // folded into the running maximum.  A piece without keys has lse = -inf and weight 0; what its row holds is
+  // never used.
+  float M = -INFINITY, L = 0.f;
   float4 acc = {0.f, 0.f, 0.f, 0.f};
-  float L = 0.f;
-  if (M > -INFINITY) {
-    for (int s0 = 0; s0 < np; s0 += 4) {
-      float w[4];
-      float4 o[4];
+  for (int s0 = 0; s0 < np; s0 += 4) {
+    float lse[4];
+    float4 o[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const bool on = s0 + u < np;
-        const float lse = on ? m.ws_lse[R + s0 + u] : -INFINITY;
-        w[u] = lse == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(lse - M);  // empty piece: weight 0, not read
-        o[u] = w[u] > 0.f ? *reinterpret_cast<const float4*>(m.ws_o + (R + s0 + u) * kD + 4 * l)
-                          : float4{0.f, 0.f, 0.f, 0.f};
-      }
+    for (int u = 0; u < 4; ++u) {
+      const bool on = s0 + u < np;
+      lse[u] = on ? m.ws_lse[R + s0 + u] : -INFINITY;
+      o[u] = on ? *reinterpret_cast<const float4*>(m.ws_o + (R + s0 + u) * kD + 4 * l) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    const float Mn = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
+    if (Mn == -INFINITY) continue;
+    const float r = M == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(M - Mn);
+    acc.x *= r; acc.y *= r; acc.z *= r; acc.w *= r;
+    L *= r;
+    M = Mn;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        acc.x += w[u] * o[u].x; acc.y += w[u] * o[u].y; acc.z += w[u] * o[u].z; acc.w += w[u] * o[u].w;
-        L += w[u];
+    for (int u = 0; u < 4; ++u) {
+      const float w = lse[u] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(lse[u] - M);
+      if (w > 0.f) {
+        acc.x += w * o[u].x; acc.y += w * o[u].y; acc.z += w * o[u].z; acc.w += w * o[u].w;
+        L += w;
       }
     }
   }
