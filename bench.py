@@ -26,7 +26,7 @@ PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 # L2-miss bytes of one launch (attention + merge kernels) of this workload under the default plan, from two
 # rocprofv3 --pmc runs (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration on a 1 GiB copy):
 # profiles/attn_fwd_kernel_c3_decode_hbm_traffic.txt
-MEASURED_TRAFFIC_BYTES = {160: 284.2e6}   # rows per request -> bytes per launch
+MEASURED_TRAFFIC_BYTES = {160: 284.4e6}   # rows per request -> bytes per launch
 
 HQ, HKV, D, PAGE = 28, 4, 128, 256
 LAYERS, N_REQ, N_CHUNKS, TOPK, CHUNK_TOKENS = 28, 8, 32, 8, 512
@@ -130,9 +130,16 @@ def cpu_baseline(torch, w, sample_layers=8):
     return sorted(times)[1] / n, cores, ref0, n
 
 
-def _time_us(torch, fn, iters=10, warmup=2):
-    for _ in range(warmup):
+def _time_us(torch, fn, iters=10, warmup=2, warm_seconds=0.05):
+    """Average launch-to-launch time of fn.  The secondary shapes run after the CPU leg, on an idle GPU whose clocks
+    have dropped: besides the `warmup` calls fn is repeated for warm_seconds before the timed calls."""
+    t0 = time.perf_counter()
+    n = 0
+    while n < warmup or time.perf_counter() - t0 < warm_seconds:
         fn()
+        n += 1
+        if n % 4 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
@@ -152,9 +159,9 @@ def secondary_shapes(torch, ops, dev):
     # response-only block (the reference engine's real decode shape, 32 rows): the HBM-bound case
     w32 = build_workload(torch, dev, q_len=32, layers=4)
     p32 = prepare(ops, w32)
-    _, g32 = time_steps(torch, p32, 16, 2)
+    _, g32 = time_steps(torch, p32, 32, 200)   # 200 warm-up steps of 4 layers = 40 ms: the clocks are up again
     b32, f32_ = algorithmic_work(32, w32["ctx"], w32["n_req"])
-    l32 = g32 / (16 * 4)
+    l32 = g32 / (32 * 4)
     out["decode_32_rows"] = {"us_per_launch": l32 * 1e6, "us_per_step_28_layers": l32 * 28e6,
                              "hbm_GBps": b32 / l32 / 1e9, "hbm_frac": b32 / l32 / 1e9 / PEAK_HBM_GBS,
                              "bf16_TFLOPs": f32_ / l32 / 1e12}
@@ -249,7 +256,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=32)
-    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--warmup", type=int, default=16)   # 16 steps = 55 ms: the GPU clocks need about 50 ms to settle
     ap.add_argument("--rows-per-group", type=int, default=0, help="override the row-group size (tuning)")
     ap.add_argument("--num-splits", type=int, default=0, help="override the KV split count (tuning)")
     ap.add_argument("--tiles-per-wg", type=int, default=0, help="override the tiles per workgroup (tuning)")
