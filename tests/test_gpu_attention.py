@@ -451,3 +451,61 @@ def test_seeded_random_shapes_and_plans(dev):
         ref = oracle_case(case, mask_mode=mode)
         err = (out - ref).abs().max().item()
         assert torch.isfinite(out).all() and err <= TOL_BF16, f"case {i} {case.meta} plan {plan} mask {mode}: max abs err {err}"
+
+
+def test_decode_step_replays_from_a_hip_graph(dev):
+    """The library allocates nothing and never synchronises, so a denoise step (slot-table build + the layers'
+    attention and merge launches) can be captured once and replayed: three replays with new queries and a new chunk
+    selection written into the same buffers in between, each compared bit for bit with the eager launches."""
+    ops = _ops()
+    case = configs.config3_small(seed=21, n_req=3)
+    d = lambda t: t.to(dev)
+    rp, rs, rl, mr = (x.to(dev) if torch.is_tensor(x) else x for x in case.range_tensors())
+    layers = 3
+    gen = torch.Generator().manual_seed(5)
+    qs = [d(case.q.clone()) for _ in range(layers)]
+    table = ops.new_slot_table(3, case.max_ctx, dev)
+    kc, vc, kn, vn, bt, qsl = d(case.k_cache), d(case.v_cache), d(case.k_new), d(case.v_new), d(case.block_table), d(case.q_start_loc)
+    preps = [ops.PreparedAttention(qs[l], kn, vn, kc, vc, bt, qsl, max_q_len=case.max_q, max_ctx_len=case.max_ctx,
+                                   ranges=(rp, rs, rl, mr), slot_table=table) for l in range(layers)]
+
+    def step():
+        preps[0].build_slot_table()
+        for p in preps:
+            p.run()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    starts = preps[0]._keep[7][1]                # the int32 range_start tensor the descriptors point at
+    base_starts = starts.clone()
+    for rep in range(3):
+        for l in range(layers):
+            qs[l].copy_((torch.randn(case.q.shape, generator=gen) / 11.3).to(torch.bfloat16))
+        # another selection: rotate the chunk starts of every request
+        for p in preps:
+            p._keep[7][1].copy_(torch.roll(base_starts, rep + 1))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = [p.out.clone() for p in preps]
+        for p in preps:
+            p.out.zero_()
+        step()
+        torch.cuda.synchronize()
+        for l in range(layers):
+            assert torch.equal(replayed[l], preps[l].out), (rep, l)
+        # and the eager result is the oracle's for the current selection
+        sel = p._keep[7][1].cpu().tolist()
+        lens = rl.cpu().tolist()
+        ptr = rp.cpu().tolist()
+        ranges = [[(sel[i], lens[i]) for i in range(ptr[r], ptr[r + 1])] for r in range(3)]
+        ref = ref_ops.sparse_decode_attention(qs[0].cpu(), case.k_new, case.v_new, case.k_cache, case.v_cache,
+                                              case.block_table, case.q_start_loc, ranges)
+        check(preps[0].out.float().cpu(), ref)
