@@ -509,3 +509,44 @@ def test_decode_step_replays_from_a_hip_graph(dev):
         ref = ref_ops.sparse_decode_attention(qs[0].cpu(), case.k_new, case.v_new, case.k_cache, case.v_cache,
                                               case.block_table, case.q_start_loc, ranges)
         check(preps[0].out.float().cpu(), ref)
+
+
+def test_seeded_random_ragged_requests_cut_ranges_and_dense_masks(dev):
+    """30 seeded random cases on top of the shapes above: requests of different lengths, selections of different
+    sizes, a range that starts inside a chunk, and random dense masks over the active rows."""
+    import random
+    rnd = random.Random(77)
+    heads = [(28, 4), (32, 32), (8, 8), (16, 2), (4, 4), (32, 1), (12, 4)]
+    for i in range(30):
+        Hq, Hkv = rnd.choice(heads)
+        n_req, n_chunks = rnd.randint(1, 7), rnd.randint(2, 8)
+        q_len = rnd.choice([7, 32, 33, 64, 96, 129, 160])
+        if Hq // Hkv * q_len > 2048:
+            q_len = 32
+        case = configs.chunked_prefix_case(5000 + i, n_req=n_req, n_chunks=n_chunks,
+                                           chunk_tokens=rnd.choice([17, 100, 255, 256, 300, 513]),
+                                           topk=rnd.randint(1, n_chunks), q_len=q_len, Hq=Hq, Hkv=Hkv,
+                                           fp8=rnd.random() < 0.3, shared_prefix=rnd.random() < 0.5)
+        lens = [rnd.randint(1, q_len) for _ in range(n_req)]
+        keep = torch.cat([torch.arange(r * q_len, r * q_len + lens[r]) for r in range(n_req)])
+        case.q, case.k_new, case.v_new = case.q[keep], case.k_new[keep], case.v_new[keep]
+        case.q_start_loc = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+        for r in range(n_req):
+            if rnd.random() < 0.5 and len(case.ranges[r]) > 1:
+                case.ranges[r] = case.ranges[r][:rnd.randint(1, len(case.ranges[r]))]
+            if rnd.random() < 0.3:
+                a0, l0 = case.ranges[r][0]
+                cut = rnd.randint(0, l0 - 1)
+                case.ranges[r][0] = (a0 + cut, l0 - cut)
+        mode, mask = rnd.choice(["full", "causal"]), None
+        if rnd.random() < 0.4:
+            n_tok = case.q.shape[0]
+            mask = torch.rand(n_tok, n_tok, generator=torch.Generator().manual_seed(i)) < 0.6
+            mask |= torch.eye(n_tok, dtype=torch.bool)
+            mode = "dense"
+        plan = rnd.choice([{}, {}, dict(rows_per_group=rnd.choice([32, 64, 128, 256])),
+                           dict(rows_per_group=128, tiles_per_workgroup=rnd.randint(1, 9))])
+        out = run_case(case, dev, mask_mode=mode, mask=mask, **plan)
+        ref = oracle_case(case, mask_mode=mode, mask=mask)
+        err = (out - ref).abs().max().item()
+        assert torch.isfinite(out).all() and err <= TOL_BF16, f"case {i} lens {lens} plan {plan} mask {mode}: max abs err {err}"
