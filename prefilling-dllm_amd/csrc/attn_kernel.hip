@@ -1324,7 +1324,7 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   const long units = (long)d->n_req * d->num_kv_heads;
   const bool fp8 = !prefill && d->k_cache != nullptr && d->max_ctx_len > 0 && d->kv_dtype == PDLLM_KV_FP8_E4M3;
   const int cus = 256;
-  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 1.5, kWide = 1.3;
+  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 1.5, kWide = 1.25;
   constexpr int kStaticLds = 66 * 1024;
   static const int js[] = {1, 2, 4, 5, 6, 8};
   static const double upw[] = {0.45, 0.75, 1.0, 1.25, 1.5, 1.0};
