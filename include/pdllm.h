@@ -381,11 +381,12 @@ enum { PDLLM_ANCHOR_SEL_NONE = 0, PDLLM_ANCHOR_SEL_REPLACE = 1, PDLLM_ANCHOR_SEL
  * base, dense, out: bf16 [n_rows, row_elems] (row strides in elements); only the anchor rows of dense
  * are read.  sel: bf16 [n_sel_rows, row_elems] indexed by the local anchor row (rows >= n_sel_rows read
  * as zero and are not valid), valid[a] = sel_counts == NULL || sel_counts[a] > 0; selection modes take
- * one sequence (n_req == 1).  out must not alias base or dense.  row_elems % 8 == 0. */
+ * one sequence (n_req == 1).  out must not alias base or dense.  row_elems % 8 == 0.  n_rows = rows of base,
+ * dense and out: a sequence that does not lie inside them is skipped. */
 int pdllm_anchor_delta_add(const void* base, int64_t base_stride, const void* dense, int64_t dense_stride,
                            const void* sel, int64_t sel_stride, int64_t n_sel_rows, const int64_t* sel_counts,
                            void* out, int64_t out_stride, const int32_t* q_start_loc, int64_t n_req,
-                           int64_t max_q_len, int64_t row_elems, int32_t stride, int32_t anchor_offset,
+                           int64_t max_q_len, int64_t n_rows, int64_t row_elems, int32_t stride, int32_t anchor_offset,
                            int32_t left, int32_t right, int32_t direction, float scale, float sel_scale,
                            int32_t sel_mode, pdllm_stream_t stream);
 

@@ -82,8 +82,8 @@ SIGNATURES = {
     "pdllm_denoise_unmask": (C.c_int, [vp, i64, vp, i64, i64, i64, i64, i32, vp, i64, f32, vp, i64, vp, vp, vp, vp, vp]),
     "pdllm_chunk_select": (C.c_int, [vp, i64, vp, i64, i64, i64, i32, i64, i32, vp, i64, vp, vp, vp, vp]),
     "pdllm_rope_inplace": (C.c_int, [vp, i64, vp, vp, i64, i64, i32, i32, vp]),
-    "pdllm_anchor_delta_add": (C.c_int, [vp, i64, vp, i64, vp, i64, i64, vp, vp, i64, vp, i64, i64, i64, i32, i32, i32,
-                                         i32, i32, f32, f32, i32, vp]),
+    "pdllm_anchor_delta_add": (C.c_int, [vp, i64, vp, i64, vp, i64, i64, vp, vp, i64, vp, i64, i64, i64, i64, i32, i32,
+                                         i32, i32, i32, f32, f32, i32, vp]),
 }
 
 

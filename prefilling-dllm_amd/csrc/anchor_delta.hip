@@ -20,7 +20,7 @@ struct AnchorParams {
   const int64_t* sel_counts;
   __bf16* out;
   const int* q_start_loc;
-  long base_stride, dense_stride, sel_stride, out_stride, n_sel_rows;
+  long base_stride, dense_stride, sel_stride, out_stride, n_sel_rows, n_rows;
   int n_req, max_q_len, groups;  // groups = row_elems / 8
   int stride, offset, lo_reach, hi_reach;  // a row r takes anchors in [r - lo_reach, r + hi_reach]
   int sel_mode;                            // 0 none, 1 replace, 2 add
@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void anchor_delta_add_kernel(const AnchorParam
   const int e = (int)(rem - (long)i * p.groups) * 8;
   const int q0 = p.q_start_loc[req];
   const int L = p.q_start_loc[req + 1] - q0;
-  if (i >= L) return;
+  if (i >= L || q0 < 0 || (long)q0 + L > p.n_rows) return;  // a sequence outside the tensors is left alone
   const bf16x8 b = *reinterpret_cast<const bf16x8*>(p.base + (long)(q0 + i) * p.base_stride + e);
   float corr[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   int a_lo = i - p.lo_reach;
@@ -89,7 +89,8 @@ using namespace pdllm;
 extern "C" int pdllm_anchor_delta_add(const void* base, int64_t base_stride, const void* dense, int64_t dense_stride,
                                       const void* sel, int64_t sel_stride, int64_t n_sel_rows,
                                       const int64_t* sel_counts, void* out, int64_t out_stride,
-                                      const int32_t* q_start_loc, int64_t n_req, int64_t max_q_len, int64_t row_elems,
+                                      const int32_t* q_start_loc, int64_t n_req, int64_t max_q_len, int64_t n_rows,
+                                      int64_t row_elems,
                                       int32_t stride, int32_t anchor_offset, int32_t left, int32_t right,
                                       int32_t direction, float scale, float sel_scale, int32_t sel_mode,
                                       pdllm_stream_t stream) {
@@ -98,7 +99,7 @@ extern "C" int pdllm_anchor_delta_add(const void* base, int64_t base_stride, con
   if (direction < PDLLM_ANCHOR_LEFT || direction > PDLLM_ANCHOR_BOTH) return PDLLM_ERR_DTYPE;
   if (sel_mode != PDLLM_ANCHOR_SEL_REPLACE && !dense) return PDLLM_ERR_NULL;
   if (sel_mode != PDLLM_ANCHOR_SEL_NONE && (!sel || n_sel_rows < 0)) return PDLLM_ERR_NULL;
-  if (n_req < 0 || max_q_len < 0 || row_elems <= 0 || row_elems % 8 || stride <= 0 || anchor_offset < 0 ||
+  if (n_req < 0 || max_q_len < 0 || n_rows < 0 || row_elems <= 0 || row_elems % 8 || stride <= 0 || anchor_offset < 0 ||
       anchor_offset >= stride || left < 0 || right < 0)
     return PDLLM_ERR_SHAPE;
   if (sel_mode != PDLLM_ANCHOR_SEL_NONE && n_req > 1) return PDLLM_ERR_UNSUPPORTED;  // selection rows are per sequence
@@ -120,6 +121,7 @@ extern "C" int pdllm_anchor_delta_add(const void* base, int64_t base_stride, con
   p.q_start_loc = q_start_loc;
   p.base_stride = base_stride; p.dense_stride = dense_stride; p.sel_stride = sel_stride; p.out_stride = out_stride;
   p.n_sel_rows = n_sel_rows;
+  p.n_rows = n_rows;
   p.n_req = (int)n_req; p.max_q_len = (int)max_q_len; p.groups = (int)(row_elems / 8);
   p.stride = stride; p.offset = anchor_offset;
   // window of anchor a: left [a - left, a], right [a, a + right], both [a - left, a + right]

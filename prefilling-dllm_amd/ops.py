@@ -888,7 +888,7 @@ def anchor_delta_add(base: torch.Tensor, dense: Optional[torch.Tensor], q_start_
     qsl = q_start_loc.to(torch.int32).contiguous()
     check(lib.pdllm_anchor_delta_add(b2.data_ptr(), b2.stride(0), _ptr(d2), d_stride, _ptr(s2), s_stride, s_rows,
                                      _ptr(cnt), out.data_ptr(), out.stride(0), qsl.data_ptr(), qsl.numel() - 1,
-                                     int(max_q_len), row_elems, int(stride), int(anchor_offset), int(left), int(right),
+                                     int(max_q_len), rows, row_elems, int(stride), int(anchor_offset), int(left), int(right),
                                      int(direction), float(scale), float(sel_scale), mode, _stream(base)),
           "anchor_delta_add")
     return out.view(base.shape)

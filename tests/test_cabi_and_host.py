@@ -80,13 +80,13 @@ def test_argument_errors_are_reported_without_a_gpu():
     ada = lib.pdllm_anchor_delta_add
     big = (ctypes.c_char * 256)()
     o = (ctypes.addressof(big) + 15) & ~15
-    assert ada(None, 128, p, 128, None, 0, 0, None, o, 128, p, 1, 4, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == -1
-    assert ada(p, 128, None, 128, None, 0, 0, None, o, 128, p, 1, 4, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == -1  # no dense
-    assert ada(p, 128, p, 128, None, 0, 0, None, o, 128, p, 1, 4, 128, 4, 4, 3, 0, 0, 1.0, 1.0, 0, None) == -2   # offset >= stride
-    assert ada(p, 128, p, 128, None, 0, 0, None, o, 128, p, 1, 4, 100, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == -2   # row_elems % 8
-    assert ada(p, 128, p, 128, None, 0, 0, None, p, 128, p, 1, 4, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == -3   # out aliases base
-    assert ada(p, 128, p, 128, p, 128, 4, None, o, 128, p, 2, 4, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 2, None) == -7    # selection, 2 sequences
-    assert ada(p, 128, p, 128, None, 0, 0, None, o, 128, p, 0, 4, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == 0    # nothing to do
+    assert ada(None, 128, p, 128, None, 0, 0, None, o, 128, p, 1, 4, 4, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == -1
+    assert ada(p, 128, None, 128, None, 0, 0, None, o, 128, p, 1, 4, 4, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == -1  # no dense
+    assert ada(p, 128, p, 128, None, 0, 0, None, o, 128, p, 1, 4, 4, 128, 4, 4, 3, 0, 0, 1.0, 1.0, 0, None) == -2   # offset >= stride
+    assert ada(p, 128, p, 128, None, 0, 0, None, o, 128, p, 1, 4, 4, 100, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == -2   # row_elems % 8
+    assert ada(p, 128, p, 128, None, 0, 0, None, p, 128, p, 1, 4, 4, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == -3   # out aliases base
+    assert ada(p, 128, p, 128, p, 128, 4, None, o, 128, p, 2, 4, 8, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 2, None) == -7    # selection, 2 sequences
+    assert ada(p, 128, p, 128, None, 0, 0, None, o, 128, p, 0, 4, 0, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == 0    # nothing to do
 
 
 def test_attention_plan_is_host_only():
