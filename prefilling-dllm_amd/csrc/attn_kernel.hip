@@ -471,6 +471,15 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
   const unsigned kn_row16 = (unsigned)((p.kn_stride * 2) >> 4);
   const unsigned vn_row16 = (unsigned)((p.vn_stride * 2) >> 4);
   int nslot[kDmaGroups];
+  // the same for a tile known to be a whole tile of the prefix / of the active block
+  auto load_slots_ctx = [&](int t) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < kDmaGroups; ++i) nslot[i] = tbl[t * kKT + 4 * NW * i + lane_row];
+  };
+  auto load_slots_new = [&](int t) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < kDmaGroups; ++i) nslot[i] = (t - Tc) * kKT + 4 * NW * i + lane_row;
+  };
   auto load_slots = [&](int t) __attribute__((always_inline)) {
     if (t < Tc) {
 #pragma unroll
@@ -713,23 +722,26 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
               (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
         }
       };
-      auto issue_k1 = [&](int t, int buf, int i) __attribute__((always_inline)) {
-        const bool ctx = t < Tc;
+      // src_tag: 0 = decide by the tile number, 1 = the tile is known to come from the cache, 2 = from the new rows
+      auto issue_k1 = [&](int t, int buf, int i, auto src_tag) __attribute__((always_inline)) {
+        constexpr int SRC = decltype(src_tag)::value;
+        const bool ctx = SRC == 1 || (SRC == 0 && t < Tc);
         copy_row(ctx ? kc_base : kn_base, ctx ? cache_row16 : kn_row16, nslot[i],
                  lds + buf * kBufBytes + wave * 1024 + i * (NW * 1024));
       };
-      auto issue_v1 = [&](int t, int buf, int i) __attribute__((always_inline)) {
-        const bool ctx = t < Tc;
+      auto issue_v1 = [&](int t, int buf, int i, auto src_tag) __attribute__((always_inline)) {
+        constexpr int SRC = decltype(src_tag)::value;
+        const bool ctx = SRC == 1 || (SRC == 0 && t < Tc);
         copy_row(ctx ? vc_base : vn_base, ctx ? cache_row16 : vn_row16, nsv[i],
                  lds + buf * kBufBytes + kTileBytes + wave * 1024 + i * (NW * 1024));
       };
       auto issue_k = [&](int t, int buf) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < kDmaGroups; ++i) issue_k1(t, buf, i);
+        for (int i = 0; i < kDmaGroups; ++i) issue_k1(t, buf, i, std::integral_constant<int, 0>{});
       };
       auto issue_v = [&](int t, int buf) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < kDmaGroups; ++i) issue_v1(t, buf, i);
+        for (int i = 0; i < kDmaGroups; ++i) issue_v1(t, buf, i, std::integral_constant<int, 0>{});
       };
       // K fragment read of QK step stp / V^T fragment read of PV step stp; ka and va point into the
       // buffer in use and move to the other one after every tile
@@ -757,17 +769,22 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
       // one iteration: softmax of tile t (scores in Sc) interleaved with QK of tile t + 1 (into Sn),
       // then PV of tile t.  PAR = buffer of V(t); K(t+1) sits in the other buffer.
       int flip = kBufBytes;  // ka: buffer 1 -> 0 -> 1 ..., va: buffer 0 -> 1 -> 0 ...
-      auto iter = [&](int t, int PAR, f32x16 (&Sc)[2]) __attribute__((always_inline)) {
-        const bool has_next = t + 1 < T1;
+      // steady (mode 1 / 2): tiles t .. t + 3 are whole tiles of the prefix / of the active block, lie inside this
+      // piece, and tile t needs no mask for any row -- every copy comes from one tensor, nothing to mask, no
+      // end-of-piece cases (the same code with those decisions made at compile time)
+      auto iter = [&](int t, int PAR, f32x16 (&Sc)[2], auto steady_tag) __attribute__((always_inline)) {
+        constexpr int MODE = decltype(steady_tag)::value;
+        constexpr bool STEADY = MODE != 0;
+        const bool has_next = STEADY || t + 1 < T1;
         // The copies of V(t+1) (slots in nsv) and K(t+2) (slots in nslot) are handed out one per
         // second step of the QK loop below: a burst would block the wave on the memory pipeline.
-        const bool k_on = t + 2 < T1;
-        if (has_next) build_mask(t + 1, PAR ^ 1);
+        const bool k_on = STEADY || t + 2 < T1;
+        if (!STEADY && has_next) build_mask(t + 1, PAR ^ 1);
 
-        const bool active = t >= Tc;
+        const bool active = !STEADY && t >= Tc;
         const int a0 = active ? (t - Tc) * kKT : 0;
-        int nvalid = active ? Sa - a0 : ctx_total - t * kKT;
-        const bool generic = nvalid < kKT || (active && p.mask_mode != PDLLM_MASK_FULL);
+        int nvalid = STEADY ? kKT : active ? Sa - a0 : ctx_total - t * kKT;
+        const bool generic = !STEADY && (nvalid < kKT || (active && p.mask_mode != PDLLM_MASK_FULL));
         nvalid = nvalid < kKT ? nvalid : kKT;
         // ---- masks, row maximum, lazy rescale (vector unit only) ----
         if (generic) {
@@ -867,14 +884,16 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
             }
             if (stp + PF < NS) rdk(kf[stp % PF], stp + PF);
             if ((stp & 1) == 1 && ((stp & 7) >> 1) < kDmaGroups) {
-              if (stp < 8) issue_v1(t + 1, PAR ^ 1, (stp & 7) >> 1);
-              else if (k_on) issue_k1(t + 2, PAR, (stp & 7) >> 1);
+              if (stp < 8) issue_v1(t + 1, PAR ^ 1, (stp & 7) >> 1, steady_tag);
+              else if (k_on) issue_k1(t + 2, PAR, (stp & 7) >> 1, steady_tag);
             }
             __builtin_amdgcn_sched_barrier(0);
           }
 #pragma unroll
           for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
-          if (t + 3 < T1) load_slots(t + 3);
+          if (MODE == 1) load_slots_ctx(t + 3);
+          else if (MODE == 2) load_slots_new(t + 3);
+          else if (t + 3 < T1) load_slots(t + 3);
         } else {
 #pragma unroll
           for (int stp = 0; stp < NS; ++stp) exp_pair(stp);
@@ -948,7 +967,23 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
       for (int ks = 0; ks < 8; ++ks) ka[ks] += kBufBytes;
       __builtin_amdgcn_s_waitcnt(0x0F70);
       __syncthreads();
-      for (int t = T0; t < T1; ++t) iter(t, (t - T0) & 1, SX);
+      {
+        using Generic = std::integral_constant<int, 0>;
+        const int whole_ctx = ctx_total / kKT;  // tiles of the prefix without a ragged end
+        const int ctx_end = (T1 < whole_ctx ? T1 : whole_ctx) - 3;
+        // active tiles that are whole and visible to every row of this row group
+        int open_tiles = Sa / kKT;
+        if (p.mask_mode == PDLLM_MASK_CAUSAL) open_tiles = (tq_first + 1) / kKT < open_tiles ? (tq_first + 1) / kKT : open_tiles;
+        if (p.mask_mode == PDLLM_MASK_DENSE) open_tiles = 0;
+        int new_end = Tc + Sa / kKT - 3;
+        new_end = new_end < T1 - 3 ? new_end : T1 - 3;
+        new_end = new_end < Tc + open_tiles ? new_end : Tc + open_tiles;
+        int t = T0;
+        for (; t < ctx_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 1>{});
+        for (; t < T1 && t < Tc; ++t) iter(t, (t - T0) & 1, SX, Generic{});
+        for (; t < new_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 2>{});
+        for (; t < T1; ++t) iter(t, (t - T0) & 1, SX, Generic{});
+      }
       // leave ka / va pointing at buffer 0 for the next piece
       if (flip > 0) {
 #pragma unroll
