@@ -979,9 +979,11 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
         new_end = new_end < T1 - 3 ? new_end : T1 - 3;
         new_end = new_end < Tc + open_tiles ? new_end : Tc + open_tiles;
         int t = T0;
-        for (; t < ctx_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 1>{});
-        for (; t < T1 && t < Tc; ++t) iter(t, (t - T0) & 1, SX, Generic{});
-        for (; t < new_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 2>{});
+        if constexpr (BUF) {  // (the wide-address form keeps the one general loop: it has no registers to spare)
+          for (; t < ctx_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 1>{});
+          for (; t < T1 && t < Tc; ++t) iter(t, (t - T0) & 1, SX, Generic{});
+          for (; t < new_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 2>{});
+        }
         for (; t < T1; ++t) iter(t, (t - T0) & 1, SX, Generic{});
       }
       // leave ka / va pointing at buffer 0 for the next piece
