@@ -26,7 +26,7 @@ PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 # L2-miss bytes of one launch (attention + merge kernels) of this workload under the default plan, from two
 # rocprofv3 --pmc runs (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration on a 1 GiB copy):
 # profiles/attn_fwd_kernel_c3_decode_hbm_traffic.txt
-MEASURED_TRAFFIC_BYTES = {160: 284.4e6}   # rows per request -> bytes per launch
+MEASURED_TRAFFIC_BYTES = {160: 272.9e6}   # rows per request -> bytes per launch
 
 HQ, HKV, D, PAGE = 28, 4, 128, 256
 LAYERS, N_REQ, N_CHUNKS, TOPK, CHUNK_TOKENS = 28, 8, 32, 8, 512
