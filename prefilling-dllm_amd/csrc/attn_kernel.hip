@@ -495,8 +495,9 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
   };
   // The whole copy of a tile is issued in one burst at the start of the tile before (handing the
   // copy instructions out between the MFMAs measured slower).
-  auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
-    const bool ctx = t < Tc;
+  // (known_ctx: the tile is known to be a tile of the prefix)
+  auto issue_tile = [&](int t, int buf, auto known_ctx) __attribute__((always_inline)) {
+    const bool ctx = decltype(known_ctx)::value || t < Tc;
     const char* kb = ctx ? kc_lane : kn_lane;
     const char* vb = ctx ? vc_lane : vn_lane;
     const unsigned kr = ctx ? cache_row16 : kn_row16;
@@ -524,8 +525,8 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
     }
   };
   // fp8: dequantise the staged rows into the LDS tile (same layout the direct copies produce)
-  auto finish_tile = [&](int t, int buf) __attribute__((always_inline)) {
-    if (KV_FP8 && t < Tc) {
+  auto finish_tile = [&](int t, int buf, auto known_ctx) __attribute__((always_inline)) {
+    if (KV_FP8 && (decltype(known_ctx)::value || t < Tc)) {
 #pragma unroll
       for (int i = 0; i < kDmaGroups; ++i) {
         char* kdst = lds + buf * kBufBytes + (i * NW + wave) * 1024 + lane * 16;
@@ -657,16 +658,20 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
     }
   };
 
-  auto compute = [&](bool generic, int t, int buf, bool has_next) __attribute__((always_inline)) {
+  // steady_tag: tiles t .. t + 2 are whole tiles of the prefix inside this piece (nothing to mask, copies from the
+  // cache, no end-of-piece cases): the same code with those decisions made at compile time
+  auto compute = [&](bool generic, int t, int buf, bool has_next, auto steady_tag) __attribute__((always_inline)) {
+    constexpr bool STEADY = decltype(steady_tag)::value;
     const int bufoff = buf * kBufBytes;
-    const bool active = t >= Tc;
+    const bool active = !STEADY && t >= Tc;
     const int a0 = active ? (t - Tc) * kKT : 0;
-    int nvalid = active ? Sa - a0 : ctx_total - t * kKT;
+    int nvalid = STEADY ? kKT : active ? Sa - a0 : ctx_total - t * kKT;
     nvalid = nvalid < kKT ? nvalid : kKT;
     using N1 = std::integral_constant<int, 1>;
     using NT = std::integral_constant<int, kNKB>;
-    if (has_next) issue_tile(t + 1, buf ^ 1);
-    if (t + 2 < T1) load_slots(t + 2);
+    if (has_next) issue_tile(t + 1, buf ^ 1, steady_tag);
+    if (STEADY) load_slots_ctx(t + 2);
+    else if (t + 2 < T1) load_slots(t + 2);
     if (HAS_A) pass(generic, NT{}, std::true_type{}, 0, bufoff, nvalid, active, a0, buf);
     if (HAS_B) {
       if (GS == 2 || ((t & 1) == parB))
@@ -674,16 +679,17 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
     }
   };
 
-  auto step = [&](int t) __attribute__((always_inline)) {
+  auto step = [&](int t, auto steady_tag) __attribute__((always_inline)) {
+    constexpr bool STEADY = decltype(steady_tag)::value;
     const int rel = t - T0;
     const int buf = rel & 1;
-    if (t + 1 < T1) build_mask(t + 1, buf ^ 1);
-    const bool active = t >= Tc;
+    if (!STEADY && t + 1 < T1) build_mask(t + 1, buf ^ 1);
+    const bool active = !STEADY && t >= Tc;
     const int a0 = active ? (t - Tc) * kKT : 0;
-    const int nv = active ? Sa - a0 : ctx_total - t * kKT;
-    const bool generic = nv < kKT || (active && p.mask_mode != PDLLM_MASK_FULL);
-    compute(generic, t, buf, t + 1 < T1);
-    if (t + 1 < T1) finish_tile(t + 1, buf ^ 1);
+    const int nv = STEADY ? kKT : active ? Sa - a0 : ctx_total - t * kKT;
+    const bool generic = !STEADY && (nv < kKT || (active && p.mask_mode != PDLLM_MASK_FULL));
+    compute(generic, t, buf, STEADY || t + 1 < T1, steady_tag);
+    if (STEADY || t + 1 < T1) finish_tile(t + 1, buf ^ 1, steady_tag);
     __syncthreads();
   };
 
@@ -1000,12 +1006,16 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
   } else
   if (T0 < T1) {
     load_slots(T0);
-    issue_tile(T0, 0);  // waits for the slots it uses
+    issue_tile(T0, 0, std::false_type{});  // waits for the slots it uses
     if (T0 + 1 < T1) load_slots(T0 + 1);
     build_mask(T0, 0);
-    finish_tile(T0, 0);
+    finish_tile(T0, 0, std::false_type{});
     __syncthreads();
-    for (int t = T0; t < T1; ++t) step(t);
+    const int whole_ctx = ctx_total / kKT;  // tiles of the prefix without a ragged end
+    const int steady_end = (T1 < whole_ctx ? T1 : whole_ctx) - 2;
+    int t = T0;
+    for (; t < steady_end; ++t) step(t, std::true_type{});
+    for (; t < T1; ++t) step(t, std::false_type{});
   }
 
   // ---- epilogue ----
