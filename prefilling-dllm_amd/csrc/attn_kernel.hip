@@ -21,9 +21,11 @@
 //   share a CU: while one waits for the matrix unit the other runs its softmax.
 //
 // Per 64-key tile
-//   K and V rows are copied HBM -> LDS by global_load_lds (16 bytes per lane, no registers);
-//   the row addresses come from a slot table that 64 threads resolve through the page table
-//   two tiles ahead.  Rows are 256 bytes = 16 chunks; chunk c of row r is stored at position
+//   K and V rows are copied HBM -> LDS without passing through registers (16 bytes per lane:
+//   buffer_load ... lds with 32-bit offsets when every tensor is below 4 GiB, global_load_lds
+//   otherwise); the row addresses come from the slot table that attn_slot_table_kernel builds
+//   from the page table and the chunk ranges once per step, read two to three tiles ahead.
+//   Rows are 256 bytes = 16 chunks; chunk c of row r is stored at position
 //   c ^ rotl4(r & 15), which makes the 128-bit K operand reads and the transposing
 //   ds_read_b64_tr_b16 V operand reads bank-conflict free.
 //   S^T = K Q^T and O^T += V^T P^T use v_mfma_f32_32x32x16_bf16; in the S^T accumulator
@@ -34,6 +36,9 @@
 //   advanced (and O rescaled) when a tile exceeds it by more than 2^8, which removes most
 //   rescale work without changing the result.
 //   fp8 e4m3 pages are dequantised (x * scale[page]) in registers while staging.
+//   The tile loops exist in a general form and in "steady" forms for runs of whole, unmasked
+//   tiles from one source, in which the mask, end-of-piece and copy-source decisions are
+//   compile-time constants (a third fewer instructions per tile).
 
 #include <type_traits>
 
