@@ -59,13 +59,17 @@ int pdllm_kv_store(const void* key, const void* value, void* k_cache, void* v_ca
 
 /* fp8 variant of the store (no reference counterpart beyond the scalar-scale
  * branch of OPS/prefix_prefill.py:118-121): quantises bf16 rows to e4m3 with
- * the scale of the destination page, x_q = e4m3(x / scale[page]).
- * k_scale/v_scale: [n_pages] fp32, already filled by the caller. */
+ * the scale of the destination page and KV head,
+ *   x_q = e4m3(x / scale[page * scale_page_stride + head * scale_head_stride]),  head = element / head_dim,
+ * the addressing pdllm_attn_desc uses to dequantise (scale_page_stride / scale_head_stride there): strides
+ * (0, 0) = one scalar as the reference passes, (1, 0) = scale[n_pages], (Hkv, 1) = scale[n_pages, Hkv].
+ * The scales are fp32, already filled by the caller, and cover every page a slot can name. */
 int pdllm_kv_store_fp8(const void* key, const void* value, void* k_cache, void* v_cache,
                        const float* k_scale, const float* v_scale,
                        const int32_t* slot_mapping, int64_t n_tokens, int64_t row_elems,
                        int64_t key_stride, int64_t value_stride, int64_t n_slots,
-                       int32_t page_size, pdllm_stream_t stream);
+                       int32_t page_size, int32_t head_dim, int64_t scale_page_stride,
+                       int64_t scale_head_stride, pdllm_stream_t stream);
 
 /* Replaces the slot-mapping builders ENG:331-351, 434-441:
  * slot[i] = page_ids[(start_token+i) / page_size] * page_size + (start_token+i) % page_size.
@@ -99,7 +103,9 @@ typedef struct pdllm_attn_desc {
   const void* v_cache;
   const float* k_scale; /* fp8 only: scale[page*scale_page_stride + kvh*scale_head_stride] */
   const float* v_scale;
-  const int32_t* block_table; /* [n_req, bt_stride] page ids (entries < 0 or >= n_pages read as zero rows) */
+  const int32_t* block_table; /* [n_req, bt_stride] page ids.  Every page a visible range touches must hold a
+                                 valid id: an entry outside [0, n_pages) is clamped into the cache (never read out
+                                 of bounds), its keys then count like any others */
   const int32_t* q_start_loc; /* [n_req+1] first active row of each request     */
   /* visible prefix of request r = ranges range_ptr[r] .. range_ptr[r+1]-1, each a
    * run of logical tokens [range_start, range_start+range_len) that is mapped

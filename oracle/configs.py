@@ -144,3 +144,47 @@ def unmask_logits(seed: int, n_seqs: int = 4, block_len: int = 32, vocab: int = 
             idx = int(torch.randint(0, vocab, (1,), generator=gen))
             logits[b, r, idx] += 30.0 if i < peaks else 14.0
     return logits.to(torch.bfloat16).reshape(n_seqs * block_len, vocab)
+
+
+def staircase_case(seed: int, *, n_req: int = 2, n_chunks: int = 4, topk: int = 3, q_len: int = 40, gran: int = 64,
+                   Hq: int = 28, Hkv: int = 4, fp8: bool = False, step: float = 9.0) -> AttnCase:
+    """A case whose softmax maximum rises by about 9 log2 units from one group of `gran` visible keys to the next
+    (every tile for gran = 64, every page for gran = 256) while the values shrink by 2^-9 per group, so that every
+    group contributes a comparable share of the result: an error in the rescaling of the running accumulators, or in
+    the log-sum-exp weights of partial results, shows up at full size instead of vanishing below the last group.
+    Key group g of a request has k[..., 0] = step * g; row (token, head) has q[..., 0] in {6.5, 8, 8.5}, which with
+    sm_scale = 1/sqrt(128) gives 7.5 / 9.2 / 9.8 log2 units per group (the first stays below the kernel's lazy
+    rescale threshold of 8, the others cross it every group)."""
+    from . import ref_ops
+    case = chunked_prefix_case(seed, n_req=n_req, n_chunks=n_chunks, chunk_tokens=PAGE, topk=topk, q_len=q_len,
+                               Hq=Hq, Hkv=Hkv, shared_prefix=False)
+    kc, vc = case.k_cache.float(), case.v_cache.float()
+    vc *= math.sqrt(case.q.shape[-1])                      # values of order one at group 0
+    kn, vn = case.k_new.float(), case.v_new.float() * math.sqrt(case.q.shape[-1])
+    q = case.q.float()
+    for r in range(n_req):
+        v_idx = 0
+        for s, l in case.ranges[r]:
+            for t in range(s, s + l):
+                g = v_idx // gran
+                page, off = int(case.block_table[r][t // PAGE]), t % PAGE
+                kc[page, off, :, 0] = step * g
+                vc[page, off] *= 2.0 ** (-9 * g)
+                v_idx += 1
+        a, b = int(case.q_start_loc[r]), int(case.q_start_loc[r + 1])
+        for i in range(b - a):
+            g = (v_idx + i) // gran
+            kn[a + i, :, 0] = step * g
+            vn[a + i] *= 2.0 ** (-9 * g)
+    rows = torch.arange(q.shape[0]).view(-1, 1) + torch.arange(Hq).view(1, -1)
+    q[:, :, 0] = torch.tensor([6.5, 8.0, 8.5])[rows % 3]
+    case.q, case.k_new, case.v_new = q.to(torch.bfloat16), kn.to(torch.bfloat16), vn.to(torch.bfloat16)
+    case.k_cache, case.v_cache = kc.to(torch.bfloat16), vc.to(torch.bfloat16)
+    if fp8:
+        kq, ks = ref_ops.quantize_pages_fp8(case.k_cache)
+        vq, vs = ref_ops.quantize_pages_fp8(case.v_cache)
+        case.k_cache_ref = ref_ops.dequantize_pages_fp8(kq, ks)
+        case.v_cache_ref = ref_ops.dequantize_pages_fp8(vq, vs)
+        case.k_cache, case.v_cache, case.k_scale, case.v_scale = kq, vq, ks, vs
+    case.meta.update(gran=gran, step=step, fp8=fp8)
+    return case

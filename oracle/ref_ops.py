@@ -12,7 +12,8 @@ Every function cites the reference lines it restates.  Path shorthand (under the
   RES = prefilling_dllm_eval/fastdllm_parallelcomp.py
 
 How each function is pinned (tests/test_oracle_*.py):
-  slot mapping / store / load / gather / scatter : closed form page*P + t%P, brute-force loops,
+  slot mapping / store / load / gather / scatter / compaction / chunk-local copy : closed form page*P + t%P,
+      token-by-token loops over plain indices (overlapping source and destination pages included),
       gather(scatter(x)) == x, the reference's slot-mapping fixture (examples/mimic_data) and the
       procedures of examples/test_dllm_kv_cache_store.py:41-43, test_dllm_kv_cache_load.py:63-65
   attention : torch SDPA in fp64, V == 1 => O == 1, key permutation invariance, split/merge

@@ -54,7 +54,7 @@ SIGNATURES = {
     "pdllm_status_string": (C.c_char_p, [C.c_int]),
     "pdllm_abi_version": (C.c_int, []),
     "pdllm_kv_store": (C.c_int, [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]),
-    "pdllm_kv_store_fp8": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]),
+    "pdllm_kv_store_fp8": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, i32, i64, i64, vp]),
     "pdllm_slot_mapping": (C.c_int, [vp, i64, i64, i64, i32, vp, vp]),
     "pdllm_kv_load": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, i64, vp, vp, vp, i32, i64, i64, i32, i64, i64, i64, vp]),
     "pdllm_attn_workspace_bytes": (i64, [C.POINTER(AttnDesc)]),

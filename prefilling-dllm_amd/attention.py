@@ -54,6 +54,13 @@ class Attention(nn.Module):
         mask_mode, dense = context.mask_kind, None
         if context.block_mask is not None:
             mask_mode, dense = "dense", context.block_mask
+            if dense.dim() != 2 or dense.shape[0] != q.shape[0]:
+                raise ValueError(f"block_mask must be [rows, keys] with one row per active token, got {tuple(dense.shape)}")
+            if dense.shape[1] != q.shape[0]:
+                # the reference's decode form [Nq, sum(ctx + Sq)] (utils/context.py:85-98): keep the active columns
+                dense = self._active_columns(dense, context)
+                if dense is None:          # nothing hidden: the bidirectional block needs no mask tensor
+                    mask_mode = "full"
         if context.is_prefill:
             o = self._maybe_prefill_sparse_attention(q, k, v, context)
             if o is not None:
@@ -72,8 +79,27 @@ class Attention(nn.Module):
                                             max_q_len=int(context.max_seqlen_q), max_ctx_len=max_ctx if has_cache else 0,
                                             context_lens=context.context_lens, ranges=context.ranges,
                                             mask_mode=mask_mode, mask=dense, sm_scale=self.scale)
-            o = self._maybe_apply_decode_delta(o, q, k, v, context)
+            o = self._maybe_apply_decode_delta(o, q, k, v, context, mask_mode, dense)
         return o.view(-1, self.num_heads * self.head_dim)
+
+    @staticmethod
+    def _active_columns(mask: torch.Tensor, context: ContextForDiffusionLM):
+        """[Nq, sum(ctx_s + Sq_s)] block-diagonal decode mask of the reference -> [Nq, Nq] over the active keys
+        (None when no active key is hidden)."""
+        from .context import active_block_mask
+        if context.is_prefill or context.context_lens is None or context.cu_seqlens_q is None:
+            raise ValueError(f"block_mask of shape {tuple(mask.shape)} does not match {mask.shape[0]} active rows")
+        ctx = [int(x) for x in context.context_lens.tolist()]
+        cu = [int(x) for x in context.cu_seqlens_q.tolist()]
+        if mask.shape[1] != sum(ctx) + cu[-1]:
+            raise ValueError(f"block_mask has {mask.shape[1]} key columns, expected {cu[-1]} (active) or "
+                             f"{sum(ctx) + cu[-1]} (contexts + active)")
+        parts, col = [], 0
+        for s, c in enumerate(ctx):
+            h = cu[s + 1] - cu[s]
+            parts.append(mask[cu[s]:cu[s + 1], col:col + c + h])
+            col += c + h
+        return active_block_mask(parts)
 
     # ---- experimental corrections (default off) ----
 
@@ -84,8 +110,9 @@ class Attention(nn.Module):
         state["max_abs"] = max(float(state.get("max_abs", 0.0)), delta_abs_max)
         state["anchor_count"] = int(state.get("anchor_count", 0)) + n_anchors
 
-    def _maybe_apply_decode_delta(self, o, q, k_new, v_new, context):
-        """attention_v4.py:86-166.  The packed active rows are one sequence, as in the reference."""
+    def _maybe_apply_decode_delta(self, o, q, k_new, v_new, context, mask_mode="full", active_mask=None):
+        """attention_v4.py:86-166.  The packed active rows are one sequence, as in the reference; active_mask is the
+        [Nq, Nq] mask over the active keys (attention_v4.py:131-133 takes those columns of the block mask)."""
         state = getattr(context, "decode_delta_state", None)
         if not state or not state.get("enabled", False) or self.layer_idx < 0:
             return o
@@ -109,12 +136,11 @@ class Attention(nn.Module):
         vc.view(-1, self.num_kv_heads, self.head_dim)[:n_prompt].copy_(full_v)
         dev = q.device
         one_seq = torch.tensor([0, seq_len], dtype=torch.int32, device=dev)
-        mask_mode = "dense" if context.block_mask is not None else context.mask_kind
         dense = ops.sparse_decode_attention(q, k_new, v_new, kc, vc,
                                             torch.arange(pages, dtype=torch.int32, device=dev).view(1, -1), one_seq,
                                             max_q_len=seq_len, max_ctx_len=n_prompt,
                                             context_lens=torch.tensor([n_prompt], dtype=torch.int32, device=dev),
-                                            mask_mode=mask_mode, mask=context.block_mask, sm_scale=self.scale)
+                                            mask_mode=mask_mode, mask=active_mask, sm_scale=self.scale)
         scale = float(state.get("scale", 1.0))
         if state.get("debug", False):
             anchors = torch.arange(offset, seq_len, stride, device=dev)

@@ -43,12 +43,49 @@ class ContextForDiffusionLM:
     def __post_init__(self):
         if self.seq_lens_ts is not None and self.context_lens is not None:
             self.total_lens = self.seq_lens_ts + self.context_lens
+        if self.block_mask is None and self.seqs:
+            # the reference's form: every sequence carries its own mask (utils/context.py:69-98)
+            masks = [getattr(seq, "current_block_mask", None) for seq in self.seqs]
+            if all(m is not None for m in masks):
+                self.block_mask = active_block_mask(masks)
         if self.block_mask is not None:
             self.mask_kind = "dense"
 
     @property
     def total_num_seqs(self) -> int:
         return len(self.seqs) if self.seqs is not None else 0
+
+
+def active_block_mask(masks) -> Optional[torch.Tensor]:
+    """Per-sequence masks of the reference -> the dense [Nq, Nq] mask over the active rows that the HIP operators
+    take, or None when every active key is visible to every active row of its sequence (the "full" mode).
+
+    A sequence's mask is [..., h, w] with h active rows and w = h keys (prefill) or w = ctx + h keys (decode,
+    unified layout: the cached context in the leading columns, engine/sequence.py:489-493,
+    fastdllm_engine.py:496-503).  The reference lays them out block-diagonally (utils/context.py:73-98); so does
+    this, on the active columns only.  The cached context is always visible to the HIP kernels -- it is in every
+    mask the reference builds -- so a mask that hides a context column is refused."""
+    parts, all_visible = [], True
+    for m in masks:
+        m = m.reshape(m.shape[-2], m.shape[-1]).to(torch.bool)
+        h, w = m.shape
+        if w < h:
+            raise ValueError(f"sequence mask of {h} rows has only {w} key columns")
+        if w > h and not bool(m[:, :w - h].all()):
+            raise ValueError("a sequence mask hides cached context keys; the HIP attention always sees the "
+                             "visible prefix (pass a shorter context or other ranges instead)")
+        a = m[:, w - h:]
+        all_visible = all_visible and bool(a.all())
+        parts.append(a)
+    if all_visible:
+        return None
+    n = sum(p.shape[0] for p in parts)
+    out = torch.zeros((n, n), dtype=torch.bool, device=parts[0].device)
+    r = 0
+    for a in parts:
+        out[r:r + a.shape[0], r:r + a.shape[0]] = a
+        r += a.shape[0]
+    return out
 
 
 def get_context_diffusion_lm() -> ContextForDiffusionLM:

@@ -31,10 +31,11 @@
 //   S^T = K Q^T and O^T += V^T P^T use v_mfma_f32_32x32x16_bf16; in the S^T accumulator
 //   layout a lane holds 16 keys of one query, so softmax statistics are lane-local plus
 //   one half-wave exchange, and P^T feeds the second MFMA straight from registers.
-//   Q is multiplied by sm_scale * log2(e) once, and the S^T accumulators start at minus the
-//   running maximum, so the MFMA result is the exponent itself.  The running maximum is only
-//   advanced (and O rescaled) when a tile exceeds it by more than 2^8, which removes most
-//   rescale work without changing the result.
+//   The S^T accumulators hold the raw fp32 dot products (first MFMA of a block starts from a zero
+//   operand); the softmax scale is applied in fp32 as one fused multiply-add per score,
+//   p = 2^(sm_scale * log2(e) * s - M), like the reference scales its fp32 dot product.  The
+//   running maximum M is only advanced (and O rescaled) when a tile exceeds it by more than 2^8,
+//   which removes most rescale work without changing the result.
 //   fp8 e4m3 pages are dequantised (x * scale[page]) in registers while staging.
 //   The tile loops exist in a general form and in "steady" forms for runs of whole, unmasked
 //   tiles from one source, in which the mask, end-of-piece and copy-source decisions are
@@ -185,15 +186,16 @@ __device__ __forceinline__ void lds_wait2(T& x, T& y) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N) : "memory");
 }
 
-// Softmax update of one row block over NKB key blocks of 32 keys.  S holds the exponents in
-// log2 units relative to the running maximum M (the accumulators were started at -M, or at 0
-// while M is still -inf), in the S^T accumulator layout: element i of a lane is key
-// 8*(i/4) + 4*h + i%4 of the block.
+// Softmax update of one row block over NKB key blocks of 32 keys.  S holds the raw dot products
+// q.k (fp32, the accumulators start at zero) in the S^T accumulator layout: element i of a lane is key
+// 8*(i/4) + 4*h + i%4 of the block.  The softmax scale is applied here in fp32, as the reference
+// scales the fp32 dot product: p = 2^(c * s - M) with c = sm_scale * log2(e) > 0 and the running
+// maximum M kept in log2 units.
 // generic (wave-uniform): keys >= lim_tile (per lane: tile bound and causal bound) and keys whose
 // bit in mrow[key block] is clear are masked out.
 template <int NKB>
 __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB][2], f32x16 (&O)[4],
-                                               float& M, float& l, int h, int kb_first, bool generic,
+                                               float& M, float& l, float c, int h, int kb_first, bool generic,
                                                int lim_tile, const uint32_t* mrow) {
   if (generic) {
 #pragma unroll
@@ -215,20 +217,14 @@ __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB
   for (int b = 0; b < NKB; ++b)
 #pragma unroll
     for (int i = (b == 0 ? 2 : 0); i < 16; i += 2) mx = fmaxf(fmaxf(mx, S[b][i]), S[b][i + 1]);
-  mx = half_swap_max(mx);
-  // advance the reference maximum only when some row of the wave needs it
-  const bool need = mx > kRescaleSlack || (M == -INFINITY && mx > -INFINITY);
+  mx = half_swap_max(mx) * c;  // log2 units; -inf (nothing visible) stays -inf
+  // advance the reference maximum only when some row of the wave needs it (M = -inf: M + slack = -inf)
+  const bool need = mx > M + kRescaleSlack;
   if (__builtin_amdgcn_ballot_w64(need) != 0) {
-    const float Muse = (M == -INFINITY) ? 0.f : M;
-    const float Mn = fmaxf(M, Muse + mx);  // mx = -inf (nothing visible) keeps M
+    const float Mn = fmaxf(M, mx);
     const float alpha = (Mn == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(M - Mn);  // M = -inf -> 0
-    const float delta = ((Mn == -INFINITY) ? 0.f : Mn) - Muse;
     M = Mn;
     l *= alpha;
-#pragma unroll
-    for (int b = 0; b < NKB; ++b)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) S[b][i] -= delta;
 #pragma unroll
     for (int db = 0; db < 4; ++db) {
 #pragma unroll
@@ -236,8 +232,9 @@ __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB
       __builtin_amdgcn_sched_barrier(0);  // one accumulator block at a time through the VALU registers
     }
   }
-  // p = 2^S rounded to bf16; the row sum is taken over the rounded values, the same ones the
+  // p = 2^(c s - M) rounded to bf16; the row sum is taken over the rounded values, the same ones the
   // second MFMA multiplies with V
+  const float negM = (M == -INFINITY) ? 0.f : -M;
   const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
   float psum = 0.f;
 #pragma unroll
@@ -246,8 +243,8 @@ __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 8; e += 2) {
-        const bf16x2 pr = {(__bf16)__builtin_amdgcn_exp2f(S[b][8 * j + e]),
-                           (__bf16)__builtin_amdgcn_exp2f(S[b][8 * j + e + 1])};
+        const bf16x2 pr = {(__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(S[b][8 * j + e], c, negM)),
+                           (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(S[b][8 * j + e + 1], c, negM))};
         psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);
         P[b][j][e] = pr[0];
         P[b][j][e + 1] = pr[1];
@@ -411,9 +408,7 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       if (valid) {
-        const bf16x8 raw = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) Q[ks][e] = (__bf16)((float)raw[e] * c);
+        Q[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) Q[ks][e] = (__bf16)0.f;
@@ -557,15 +552,11 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
     float& l1 = forA ? lA : lB;
     const int srow1 = forA ? srowA : srowB;
 
-    // the accumulators start at minus the running maximum
-    const float i1 = (M1 == -INFINITY) ? 0.f : -M1;
     f32x16 S1[NKB];
 #pragma unroll
     for (int b = 0; b < NKB; ++b)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        S1[b][i] = i1;
-      }
+      for (int i = 0; i < 16; ++i) S1[b][i] = 0.f;
     if constexpr (!QLDS) {
       constexpr int PF = 4;  // operand reads run PF steps ahead of the MFMAs (LDS latency ~ 3-4 MFMAs)
       constexpr int NS = 8 * NKB;
@@ -624,7 +615,7 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
       if (causal_here) { const int cl = srow1 - a0 + 1; lim = cl < lim ? cl : lim; }
       int tl = srow1 - tq_first;
       tl = tl < 0 ? 0 : (tl >= kMaxTok ? kMaxTok - 1 : tl);
-      softmax_update<NKB>(S1, P1, O1, M1, l1, h, kb_first, generic, lim,
+      softmax_update<NKB>(S1, P1, O1, M1, l1, c, h, kb_first, generic, lim,
                           dense_here ? &s_maskbits[par][tl][0] : nullptr);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -826,19 +817,13 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
         for (int b = 0; b < 2; ++b)
 #pragma unroll
           for (int i = (b == 0 ? 2 : 0); i < 16; i += 2) mx = fmaxf(fmaxf(mx, Sc[b][i]), Sc[b][i + 1]);
-        mx = half_swap_max(mx);
-        const bool need = mx > kRescaleSlack || (MA == -INFINITY && mx > -INFINITY);
+        mx = half_swap_max(mx) * c;  // log2 units
+        const bool need = mx > MA + kRescaleSlack;
         if (__builtin_amdgcn_ballot_w64(need) != 0) {
-          const float Muse = (MA == -INFINITY) ? 0.f : MA;
-          const float Mn = fmaxf(MA, Muse + mx);
+          const float Mn = fmaxf(MA, mx);
           const float alpha = (Mn == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(MA - Mn);
-          const float delta = ((Mn == -INFINITY) ? 0.f : Mn) - Muse;
           MA = Mn;
           lA *= alpha;
-#pragma unroll
-          for (int b = 0; b < 2; ++b)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) Sc[b][i] -= delta;
 #pragma unroll
           for (int db = 0; db < 4; ++db) {
 #pragma unroll
@@ -847,18 +832,19 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
           }
         }
         // ---- exponentials of tile t, two per step, between the MFMAs of QK(t+1) ----
-        const float init = (MA == -INFINITY) ? 0.f : -MA;
+        const float negM = (MA == -INFINITY) ? 0.f : -MA;
         f32x16 Sn[2];
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) Sn[b][i] = init;
+          for (int i = 0; i < 16; ++i) Sn[b][i] = 0.f;
         bf16x8 P[2][2];
         const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
         float psum = 0.f;
         auto exp_pair = [&](int stp) __attribute__((always_inline)) {
           const int b = stp >> 3, i = 2 * (stp & 7);
-          const bf16x2 pr = {(__bf16)__builtin_amdgcn_exp2f(Sc[b][i]), (__bf16)__builtin_amdgcn_exp2f(Sc[b][i + 1])};
+          const bf16x2 pr = {(__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(Sc[b][i], c, negM)),
+                             (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(Sc[b][i + 1], c, negM))};
           psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);
           P[b][i >> 3][i & 7] = pr[0];
           P[b][i >> 3][(i & 7) + 1] = pr[1];
@@ -1342,6 +1328,7 @@ static int validate_desc(const pdllm_attn_desc* d, bool prefill) {
   if (has_cache && d->slot_table != nullptr) {
     if (d->slot_table_stride < slot_table_stride_for(d) || ((uintptr_t)d->slot_table % 4)) return PDLLM_ERR_STRIDE;
   }
+  if (!(d->sm_scale > 0.f) || !(d->sm_scale < 1e30f)) return PDLLM_ERR_SHAPE;  // the row maximum is taken before scaling
   if (d->num_splits < 0 || d->num_splits > 16 || d->tiles_per_workgroup < 0) return PDLLM_ERR_SHAPE;
   if (d->rows_per_group != 0) {
     const int j = d->rows_per_group / 32;

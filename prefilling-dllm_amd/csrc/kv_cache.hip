@@ -62,18 +62,20 @@ __global__ __launch_bounds__(256) void kv_store_fp8_kernel(
     const uint4* __restrict__ key, const uint4* __restrict__ value, uint2* __restrict__ k_cache,
     uint2* __restrict__ v_cache, const float* __restrict__ k_scale, const float* __restrict__ v_scale,
     const int* __restrict__ slot_mapping, long n_tokens, int chunks_per_row, long key_stride16,
-    long value_stride16, long n_slots, int page_shift) {
+    long value_stride16, long n_slots, int page_shift, int chunks_per_head, long scale_page_stride,
+    long scale_head_stride) {
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
   const long tok = idx / chunks_per_row;
   const int ch = (int)(idx - tok * chunks_per_row);
   if (tok >= n_tokens) return;
   const long slot = slot_mapping[tok];
   if (slot < 0 || slot >= n_slots) return;
-  const long page = slot >> page_shift;
+  // the scale of (page, KV head), addressed like the attention kernel addresses it when it dequantises
+  const long so = (slot >> page_shift) * scale_page_stride + (long)(ch / chunks_per_head) * scale_head_stride;
   const uint4 kv = key[tok * key_stride16 + ch];
   const uint4 vv = value[tok * value_stride16 + ch];
-  k_cache[slot * chunks_per_row + ch] = quant_fp8x8(kv, k_scale[page]);
-  v_cache[slot * chunks_per_row + ch] = quant_fp8x8(vv, v_scale[page]);
+  k_cache[slot * chunks_per_row + ch] = quant_fp8x8(kv, k_scale[so]);
+  v_cache[slot * chunks_per_row + ch] = quant_fp8x8(vv, v_scale[so]);
 }
 
 __global__ __launch_bounds__(256) void slot_mapping_kernel(const int* __restrict__ page_ids,
@@ -241,9 +243,12 @@ extern "C" int pdllm_kv_store_fp8(const void* key, const void* value, void* k_ca
                                   const float* k_scale, const float* v_scale,
                                   const int32_t* slot_mapping, int64_t n_tokens, int64_t row_elems,
                                   int64_t key_stride, int64_t value_stride, int64_t n_slots,
-                                  int32_t page_size, pdllm_stream_t stream) {
+                                  int32_t page_size, int32_t head_dim, int64_t scale_page_stride,
+                                  int64_t scale_head_stride, pdllm_stream_t stream) {
   if (!key || !value || !k_cache || !v_cache || !slot_mapping || !k_scale || !v_scale) return PDLLM_ERR_NULL;
   if (n_tokens < 0 || row_elems <= 0 || n_slots < 0) return PDLLM_ERR_SHAPE;
+  if (head_dim <= 0 || head_dim % 8 || row_elems % head_dim) return PDLLM_ERR_SHAPE;
+  if (scale_page_stride < 0 || scale_head_stride < 0) return PDLLM_ERR_STRIDE;
   const int shift = ilog2_exact_l(page_size);
   if (shift < 0) return PDLLM_ERR_SHAPE;
   if (row_elems % 8 || key_stride % 8 || value_stride % 8) return PDLLM_ERR_STRIDE;
@@ -256,7 +261,8 @@ extern "C" int pdllm_kv_store_fp8(const void* key, const void* value, void* k_ca
                      static_cast<hipStream_t>(stream), static_cast<const uint4*>(key),
                      static_cast<const uint4*>(value), static_cast<uint2*>(k_cache),
                      static_cast<uint2*>(v_cache), k_scale, v_scale, slot_mapping, (long)n_tokens, cpr,
-                     (long)(key_stride / 8), (long)(value_stride / 8), (long)n_slots, shift);
+                     (long)(key_stride / 8), (long)(value_stride / 8), (long)n_slots, shift, (int)(head_dim / 8),
+                     (long)scale_page_stride, (long)scale_head_stride);
   return launch_status();
 }
 

@@ -33,6 +33,25 @@ def _need_cuda(*ts: torch.Tensor) -> None:
             raise ValueError("HIP operators require device tensors (the product path has no CPU fallback).")
 
 
+def _scale_layout(k_scale: torch.Tensor, v_scale: torch.Tensor, n_pages: int, num_kv_heads: int,
+                  device) -> Tuple[int, int]:
+    """(page stride, head stride) of the fp8 scales, the same for the store and for the attention: one scalar
+    (what the reference passes, prefix_prefill.py:118-121), scale[n_pages], or scale[n_pages, Hkv]."""
+    for name, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+        if not isinstance(t, torch.Tensor) or t.dtype != torch.float32 or t.device != device:
+            raise ValueError(f"{name} must be an fp32 tensor on the device of the cache")
+    if k_scale.shape != v_scale.shape or k_scale.stride() != v_scale.stride():
+        raise ValueError("k_scale and v_scale must have the same layout")
+    if k_scale.numel() == 1:
+        return 0, 0
+    if k_scale.dim() == 1 and k_scale.shape[0] >= n_pages:
+        return k_scale.stride(0), 0
+    if k_scale.dim() == 2 and k_scale.shape[0] >= n_pages and k_scale.shape[1] == num_kv_heads:
+        return k_scale.stride(0), k_scale.stride(1)
+    raise ValueError(f"fp8 scales must be a scalar, [n_pages] or [n_pages, Hkv] with n_pages >= {n_pages}, "
+                     f"Hkv = {num_kv_heads}; got {tuple(k_scale.shape)}")
+
+
 _WORKSPACES: dict = {}
 
 
@@ -77,10 +96,14 @@ def store_kvcache_unified_layout(key: torch.Tensor, value: torch.Tensor, k_cache
         raise ValueError("unified KV cache must be contiguous")
     if k_cache.dtype == torch.float8_e4m3fn:
         if k_scale is None or v_scale is None:
-            raise ValueError("fp8 KV cache needs per-page k_scale / v_scale")
+            raise ValueError("fp8 KV cache needs k_scale / v_scale")
+        if key.dtype != torch.bfloat16 or value.dtype != torch.bfloat16:
+            raise ValueError("the fp8 store quantises bf16 rows")
+        sps, shs = _scale_layout(k_scale, v_scale, k_cache.shape[0], num_heads, k_cache.device)
         st = lib.pdllm_kv_store_fp8(key.data_ptr(), value.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                     k_scale.data_ptr(), v_scale.data_ptr(), slot_mapping.data_ptr(), N, D,
-                                    key.stride(0), value.stride(0), n_slots, k_cache.shape[1], _stream(key))
+                                    key.stride(0), value.stride(0), n_slots, k_cache.shape[1], head_dim, sps, shs,
+                                    _stream(key))
     else:
         if key.dtype != k_cache.dtype or key.element_size() != 2:
             raise ValueError("KV store expects 16-bit rows of the cache dtype")
@@ -129,14 +152,16 @@ def load_kvcache(k_cache: torch.Tensor, v_cache: torch.Tensor, context, k_new: t
     max_total = int((ctxlens + seqlens).max().item())
     k_out = torch.empty((total, h_kv, head_dim), device=k_cache.device, dtype=k_cache.dtype)
     v_out = torch.empty_like(k_out)
+    _need_cuda(context.block_tables, ctxlens, cu_q, cu_k)
+    # converted copies stay bound to locals until the call has been enqueued
     bt = context.block_tables.to(torch.int32).contiguous()
+    ctx32, cuq32, cuk32 = (t.to(torch.int32).contiguous() for t in (ctxlens, cu_q, cu_k))
     D = h_kv * head_dim
     check(lib.pdllm_kv_load(k_cache.data_ptr(), v_cache.data_ptr(), k_new.data_ptr(), v_new.data_ptr(),
                             k_out.data_ptr(), v_out.data_ptr(), bt.data_ptr(), bt.stride(0),
-                            ctxlens.to(torch.int32).contiguous().data_ptr(),
-                            cu_q.to(torch.int32).contiguous().data_ptr(),
-                            cu_k.to(torch.int32).contiguous().data_ptr(), num_seqs, max_total, D, page_size,
+                            ctx32.data_ptr(), cuq32.data_ptr(), cuk32.data_ptr(), num_seqs, max_total, D, page_size,
                             n_blocks, k_new.stride(0), D, _stream(k_cache)), "load_kvcache")
+    del bt, ctx32, cuq32, cuk32
     return k_out, v_out
 
 
@@ -181,12 +206,8 @@ def _fill_desc(q, k_new, v_new, out, k_cache, v_cache, block_table, q_start_loc,
             if k_scale is None or v_scale is None:
                 raise ValueError("fp8 KV cache needs k_scale / v_scale tensors")
             desc.k_scale, desc.v_scale = k_scale.data_ptr(), v_scale.data_ptr()
-            if k_scale.numel() == 1:
-                desc.scale_page_stride = desc.scale_head_stride = 0
-            elif k_scale.dim() == 1:
-                desc.scale_page_stride, desc.scale_head_stride = 1, 0
-            else:
-                desc.scale_page_stride, desc.scale_head_stride = k_scale.stride(0), k_scale.stride(1)
+            desc.scale_page_stride, desc.scale_head_stride = _scale_layout(k_scale, v_scale, k_cache.shape[0], Hkv,
+                                                                           k_cache.device)
         else:
             raise ValueError(f"unsupported KV cache dtype {k_cache.dtype}")
         desc.block_table, desc.bt_stride = block_table.data_ptr(), block_table.stride(0)
@@ -194,6 +215,18 @@ def _fill_desc(q, k_new, v_new, out, k_cache, v_cache, block_table, q_start_loc,
         desc.range_ptr, desc.range_start, desc.range_len = rp.data_ptr(), rs.data_ptr(), rl.data_ptr()
         desc.max_ranges = int(max_ranges)
     return desc
+
+
+def _active_mask(mask: Optional[torch.Tensor], n_tokens: int) -> Optional[torch.Tensor]:
+    """The dense mask the kernels index as mask[q_start + i, q_start + j] over the ACTIVE rows and keys only."""
+    if mask is None:
+        return None
+    if mask.dim() != 2 or tuple(mask.shape) != (n_tokens, n_tokens):
+        raise ValueError(f"mask must be [n_tokens, n_tokens] = [{n_tokens}, {n_tokens}] over the active rows and "
+                         f"active keys, got {tuple(mask.shape)}; a mask with context columns "
+                         "([Sq, ctx + Sq], the reference's decode form) goes through context.active_block_mask")
+    _need_cuda(mask)
+    return mask.to(torch.bool).contiguous().view(torch.uint8)
 
 
 def sparse_decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
@@ -214,7 +247,9 @@ def sparse_decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.T
     token ranges `ranges = (range_ptr[n_req+1], range_start[], range_len[], max_ranges)`,
     which is how a top-K chunk selection reads its non-contiguous chunks in place.
     mask_mode: "full" (bidirectional block), "causal", or "dense" with mask[n_tok, n_tok]."""
-    _need_cuda(q, k_new, v_new, q_start_loc)
+    _need_cuda(q, k_new, v_new, q_start_loc, k_cache, v_cache, block_table, context_lens, k_scale, v_scale, out)
+    if ranges is not None:
+        _need_cuda(*ranges[:3])
     n_tokens, Hq, d = q.shape
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(d)
@@ -223,8 +258,7 @@ def sparse_decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.T
     q_start_loc = q_start_loc.to(torch.int32).contiguous()
     n_req = q_start_loc.numel() - 1
     mode = {"full": _lib.MASK_FULL, "causal": _lib.MASK_CAUSAL, "dense": _lib.MASK_DENSE}[mask_mode]
-    if mask is not None:
-        mask = mask.to(torch.bool).contiguous().view(torch.uint8)
+    mask = _active_mask(mask, n_tokens)
     if k_cache is not None and max_ctx_len > 0:
         block_table = block_table.to(torch.int32).contiguous()
         if ranges is None:
@@ -261,14 +295,16 @@ class PreparedAttention:
         """slot_table: an int32 tensor from `new_slot_table` shared by every layer of a step; the caller
         refreshes it with `build_slot_table()` of any one of the prepared layers whenever the page table
         or the ranges change.  Without it every `run()` rebuilds the table in its workspace."""
-        _need_cuda(q, k_new, v_new, q_start_loc)
+        _need_cuda(q, k_new, v_new, q_start_loc, k_cache, v_cache, block_table, context_lens, k_scale, v_scale, out,
+                   workspace, slot_table)
+        if ranges is not None:
+            _need_cuda(*ranges[:3])
         n_tokens, Hq, d = q.shape
         self.out = torch.empty_like(q) if out is None else out
         q_start_loc = q_start_loc.to(torch.int32).contiguous()
         n_req = q_start_loc.numel() - 1
         mode = {"full": _lib.MASK_FULL, "causal": _lib.MASK_CAUSAL, "dense": _lib.MASK_DENSE}[mask_mode]
-        if mask is not None:
-            mask = mask.to(torch.bool).contiguous().view(torch.uint8)
+        mask = _active_mask(mask, n_tokens)
         if k_cache is not None and max_ctx_len > 0:
             block_table = block_table.to(torch.int32).contiguous()
             if ranges is None:
@@ -341,6 +377,7 @@ def attention_plan(n_req: int, num_q_heads: int, num_kv_heads: int, *, max_q_len
     desc.num_q_heads, desc.num_kv_heads, desc.head_dim = num_q_heads, num_kv_heads, d
     desc.n_req, desc.max_q_len, desc.max_ctx_len = n_req, int(max_q_len), int(max_ctx_len)
     desc.num_splits, desc.rows_per_group = num_splits, rows_per_group
+    desc.sm_scale = 1.0 / math.sqrt(d)
     rows, splits = C.c_int32(0), C.c_int32(0)
     check(lib.pdllm_attn_plan(C.byref(desc), 1 if prefill else 0, C.byref(rows), C.byref(splits)), "attention_plan")
     return rows.value, splits.value
@@ -407,6 +444,12 @@ def diffusion_lm_parallel_flash_decoding(query, key, value, output, kv_cache_dty
         mode = "full" if bidirectional else "causal"
     ks = k_scale if isinstance(k_scale, torch.Tensor) else None
     vs = v_scale if isinstance(v_scale, torch.Tensor) else None
+    if has_cache and key_cache.dtype in (torch.float8_e4m3fn, torch.uint8):
+        # the reference passes Python floats (1.0, 1.0): one scalar scale for the whole cache
+        if ks is None and k_scale is not None:
+            ks = torch.tensor(float(k_scale), dtype=torch.float32, device=key_cache.device)
+        if vs is None and v_scale is not None:
+            vs = torch.tensor(float(v_scale), dtype=torch.float32, device=key_cache.device)
     sparse_decode_attention(query, key, value, key_cache if has_cache else None,
                             value_cache if has_cache else None, block_table, qsl,
                             max_q_len=int(max_query_len), max_ctx_len=max_ctx, context_lens=ctx,
@@ -477,6 +520,9 @@ def topk_lowest_index(scores: torch.Tensor, k: int, sorted_ascending: bool = Tru
     if s2.dtype != torch.float32 or s2.stride(-1) != 1:
         s2 = s2.float().contiguous()
     rows, n = s2.shape
+    k = min(int(k), n)      # the reference takes ranked[:k] of n chunks
+    if k <= 0:
+        return torch.empty((0,) if squeeze else (rows, 0), dtype=torch.int64, device=scores.device)
     out = torch.empty((rows, k), dtype=torch.int64, device=scores.device)
     check(lib.pdllm_topk_lowest_index(s2.data_ptr(), rows, n, s2.stride(0), k, 1 if sorted_ascending else 0,
                                       out.data_ptr(), _stream(scores)), "topk_lowest_index")

@@ -72,6 +72,36 @@ def test_gather_scatter_compaction_invariants():
     assert torch.equal(cache[pages[2], 100:], before[pages[2], 100:])
 
 
+def test_chunk_local_kv_copy_token_by_token():
+    """copy_chunk_local_kv against a token-by-token loop over plain Python indices: source chunk that starts in
+    the middle of a page, destination that starts in the middle of another, source and destination page lists
+    that share pages (the copy of a head reads everything before it writes), a different keep list per head."""
+    gen = torch.Generator().manual_seed(6)
+    P, H, d = 256, 3, 4
+    cache = torch.randn(7, P, H, d, generator=gen)
+    src_pages, dst_pages = [5, 2, 6], [2, 0, 3]          # page 2 is both read and written
+    src_chunk_start, dst_start, chunk_len, keep_n = 200, 130, 500, 330
+    keep = torch.stack([torch.sort(torch.randperm(chunk_len, generator=gen)[:keep_n]).values for _ in range(H)])
+    keep[1] = torch.arange(keep_n)                        # one head keeps a plain prefix
+    before = cache.clone()
+    ref_ops.copy_chunk_local_kv(cache, src_pages, dst_pages, src_chunk_start, dst_start, keep)
+    want = before.clone()
+    for h in range(H):
+        for j in range(keep_n):
+            s = int(keep[h, j]) + src_chunk_start
+            t = dst_start + j
+            want[dst_pages[t // P], t % P, h] = before[src_pages[s // P], s % P, h]
+    assert torch.equal(cache, want)
+    # some destination slot really lay inside the source range of page 2 (the overlap is exercised) ...
+    assert any(dst_pages[(dst_start + j) // P] == 2 for j in range(keep_n))
+    assert any(src_pages[(int(keep[0, j]) + src_chunk_start) // P] == 2 for j in range(keep_n))
+    # ... and nothing outside the destination range changed
+    touched = torch.zeros(7, P, dtype=torch.bool)
+    for j in range(keep_n):
+        touched[dst_pages[(dst_start + j) // P], (dst_start + j) % P] = True
+    assert torch.equal(cache[~touched], before[~touched])
+
+
 # ---------------------------------------------------------------- attention
 
 def _sdpa64(q, k, v, mask, scale):
