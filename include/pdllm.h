@@ -31,7 +31,8 @@ enum {
   PDLLM_ERR_DTYPE = -4,       /* unknown dtype / mode enumerator                  */
   PDLLM_ERR_WORKSPACE = -5,   /* workspace missing or too small                   */
   PDLLM_ERR_LAUNCH = -6,      /* hipLaunch reported an error                      */
-  PDLLM_ERR_UNSUPPORTED = -7  /* valid request the kernels do not cover           */
+  PDLLM_ERR_UNSUPPORTED = -7, /* valid request the kernels do not cover           */
+  PDLLM_ERR_SCRATCH_LIMIT = -8 /* input too large for the static device scratch of a *_static entry point */
 };
 
 enum { PDLLM_KV_BF16 = 0, PDLLM_KV_FP8_E4M3 = 1 };
@@ -342,6 +343,24 @@ int pdllm_denoise_unmask(const void* logits, int64_t logits_stride, const void* 
                          int32_t shift, int64_t* block_ids, int64_t mask_token_id, float threshold,
                          void* workspace, int64_t workspace_bytes, float* conf_out, int64_t* token_out,
                          uint8_t* transfer_out, int32_t* n_masked_left, pdllm_stream_t stream);
+
+/* pdllm_denoise_unmask for callers that cannot allocate a workspace or have one allocated for them (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
+ * the reference.  Same arguments and results as pdllm_denoise_unmask without the workspace: the partial
+ * results of the vocabulary scan live in a static device array of PDLLM_STATIC_SCRATCH_BYTES that every GPU
+ * the library runs on holds until the process ends.  The call allocates and frees nothing.  An input whose
+ * partials do not fit, pdllm_vocab_workspace_bytes(n_seqs * block_len, vocab) > PDLLM_STATIC_SCRATCH_BYTES,
+ * is refused with PDLLM_ERR_SCRATCH_LIMIT (16384 (row, split) partials of 16 bytes fit: up to 16384 rows, i.e. 512
+ * sequences of 32 positions, of any vocabulary).
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams or threads)
+ * race; calls on one stream do not.  The first call on a device looks the array's address up; make it
+ * outside a stream capture. */
+#define PDLLM_STATIC_SCRATCH_BYTES (256 * 1024)
+int pdllm_denoise_unmask_static(const void* logits, int64_t logits_stride, const void* last_logit,
+                                int64_t last_logit_stride, int64_t n_seqs, int64_t block_len, int64_t vocab,
+                                int32_t shift, int64_t* block_ids, int64_t mask_token_id, float threshold,
+                                float* conf_out, int64_t* token_out, uint8_t* transfer_out,
+                                int32_t* n_masked_left, pdllm_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * Rotary embedding (the step in front of the path)                           *

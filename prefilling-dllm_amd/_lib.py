@@ -20,6 +20,7 @@ ERRORS = {
     -5: ("WORKSPACE", RuntimeError),
     -6: ("LAUNCH", RuntimeError),
     -7: ("UNSUPPORTED", NotImplementedError),
+    -8: ("SCRATCH_LIMIT", RuntimeError),
 }
 
 KV_BF16, KV_FP8_E4M3 = 0, 1
@@ -80,6 +81,7 @@ SIGNATURES = {
     "pdllm_rope_qk_store": (C.c_int, [vp, i64, i32, vp, i64, vp, i64, i32, i32, vp, vp, i64, i64, vp, vp, vp, i64, vp]),
     "pdllm_vote_histogram": (C.c_int, [vp, i64, i64, vp, vp]),
     "pdllm_denoise_unmask": (C.c_int, [vp, i64, vp, i64, i64, i64, i64, i32, vp, i64, f32, vp, i64, vp, vp, vp, vp, vp]),
+    "pdllm_denoise_unmask_static": (C.c_int, [vp, i64, vp, i64, i64, i64, i64, i32, vp, i64, f32, vp, vp, vp, vp, vp]),
     "pdllm_chunk_select": (C.c_int, [vp, i64, vp, i64, i64, i64, i32, i64, i32, vp, i64, vp, vp, vp, vp]),
     "pdllm_rope_inplace": (C.c_int, [vp, i64, vp, vp, i64, i64, i32, i32, vp]),
     "pdllm_anchor_delta_add": (C.c_int, [vp, i64, vp, i64, vp, i64, i64, vp, vp, i64, vp, i64, i64, i64, i64, i32, i32,

@@ -11,6 +11,7 @@ extern "C" const char* pdllm_status_string(int status) {
     case PDLLM_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
     case PDLLM_ERR_LAUNCH: return "kernel launch failed";
     case PDLLM_ERR_UNSUPPORTED: return "request not covered by the kernels";
+    case PDLLM_ERR_SCRATCH_LIMIT: return "input exceeds the static device scratch of this entry point";
     default: return "unknown status";
   }
 }

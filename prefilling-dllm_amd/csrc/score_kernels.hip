@@ -8,6 +8,8 @@
 // Reference: fastdllm_engine.py:1148-1152 (self-information), :1647-1681 (shift + confidence),
 // :2146-2157 (transfer rule) of the reference engine.
 
+#include <mutex>
+
 #include "pdllm_common.h"
 
 namespace pdllm {
@@ -554,12 +556,12 @@ extern "C" int pdllm_chunk_select(const void* logits, int64_t logits_stride, con
   return launch_status();
 }
 
-extern "C" int pdllm_denoise_unmask(const void* logits, int64_t logits_stride, const void* last_logit,
-                                    int64_t last_logit_stride, int64_t n_seqs, int64_t block_len,
-                                    int64_t vocab, int32_t shift, int64_t* block_ids, int64_t mask_token_id,
-                                    float threshold, void* workspace, int64_t workspace_bytes,
-                                    float* conf_out, int64_t* token_out, uint8_t* transfer_out,
-                                    int32_t* n_masked_left, pdllm_stream_t stream) {
+static int denoise_unmask_launch(const void* logits, int64_t logits_stride, const void* last_logit,
+                                 int64_t last_logit_stride, int64_t n_seqs, int64_t block_len,
+                                 int64_t vocab, int32_t shift, int64_t* block_ids, int64_t mask_token_id,
+                                 float threshold, void* workspace, int64_t workspace_bytes,
+                                 float* conf_out, int64_t* token_out, uint8_t* transfer_out,
+                                 int32_t* n_masked_left, pdllm_stream_t stream) {
   if (!block_ids || !conf_out || !token_out || !transfer_out) return PDLLM_ERR_NULL;
   if (n_seqs < 0 || block_len <= 0) return PDLLM_ERR_SHAPE;
   if (last_logit && last_logit_stride < vocab) return PDLLM_ERR_STRIDE;
@@ -577,6 +579,61 @@ extern "C" int pdllm_denoise_unmask(const void* logits, int64_t logits_stride, c
                      reinterpret_cast<long*>(block_ids), (long)block_len, (long)mask_token_id, threshold,
                      conf_out, reinterpret_cast<long*>(token_out), transfer_out, n_masked_left);
   return launch_status();
+}
+
+extern "C" int pdllm_denoise_unmask(const void* logits, int64_t logits_stride, const void* last_logit,
+                                    int64_t last_logit_stride, int64_t n_seqs, int64_t block_len,
+                                    int64_t vocab, int32_t shift, int64_t* block_ids, int64_t mask_token_id,
+                                    float threshold, void* workspace, int64_t workspace_bytes,
+                                    float* conf_out, int64_t* token_out, uint8_t* transfer_out,
+                                    int32_t* n_masked_left, pdllm_stream_t stream) {
+  return denoise_unmask_launch(logits, logits_stride, last_logit, last_logit_stride, n_seqs, block_len, vocab, shift,
+                               block_ids, mask_token_id, threshold, workspace, workspace_bytes, conf_out, token_out,
+                               transfer_out, n_masked_left, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same step for callers that cannot allocate a workspace: the per-row, per-split partials live
+// in a static device array.  Every GPU the library runs on holds its own copy of the array at its
+// own address; that address is looked up once per device, on the first call made with that device
+// current, and host code uses the looked-up pointer only (the array's name is not a device address
+// on the host).
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[PDLLM_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+static int static_scratch_ptr(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return PDLLM_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return PDLLM_ERR_LAUNCH;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return PDLLM_OK;
+}
+
+extern "C" int pdllm_denoise_unmask_static(const void* logits, int64_t logits_stride, const void* last_logit,
+                                           int64_t last_logit_stride, int64_t n_seqs, int64_t block_len,
+                                           int64_t vocab, int32_t shift, int64_t* block_ids,
+                                           int64_t mask_token_id, float threshold, float* conf_out,
+                                           int64_t* token_out, uint8_t* transfer_out, int32_t* n_masked_left,
+                                           pdllm_stream_t stream) {
+  if (n_seqs < 0 || block_len <= 0 || vocab <= 0) return PDLLM_ERR_SHAPE;
+  if (n_seqs == 0) return PDLLM_OK;
+  if (n_seqs * block_len > 65535) return PDLLM_ERR_UNSUPPORTED;
+  if (vocab_ws_bytes(n_seqs * block_len, vocab) > (int64_t)PDLLM_STATIC_SCRATCH_BYTES) return PDLLM_ERR_SCRATCH_LIMIT;
+  void* ptr = nullptr;
+  const int st = static_scratch_ptr(&ptr);
+  if (st != PDLLM_OK) return st;
+  // every partial the tail reads is written by the scan of the same call: nothing has to start at zero
+  return denoise_unmask_launch(logits, logits_stride, last_logit, last_logit_stride, n_seqs, block_len, vocab, shift,
+                               block_ids, mask_token_id, threshold, ptr, (int64_t)PDLLM_STATIC_SCRATCH_BYTES, conf_out,
+                               token_out, transfer_out, n_masked_left, stream);
 }
 
 extern "C" int pdllm_rope_qk_store(void* q, int64_t q_stride, int32_t num_q_heads, void* k, int64_t k_stride,
