@@ -1,0 +1,144 @@
+// Shared pieces of the attention kernels for gfx950: tile geometry, the kernel parameter block, and the
+// hand-issued LDS operand reads with their explicit wait counts.
+#pragma once
+
+#include "pdllm_common.h"
+
+namespace pdllm {
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+constexpr int kD = 128;          // head dim
+constexpr int kKT = 64;          // keys per tile
+constexpr int kNKB = kKT / 32;   // 32-key blocks per tile
+constexpr int kThreads = 256;    // 4 wavefronts (8 for the 256-row group)
+constexpr int kRowBytes = 256;   // one K or V row in LDS
+constexpr int kTileBytes = kKT * kRowBytes;      // 16384
+constexpr int kBufBytes = 2 * kTileBytes;        // K tile + V tile
+constexpr int kMainBytes = 2 * kBufBytes;        // double buffered: 65536
+constexpr int kPartBytes = kD * 32 * 4;          // LDS partial of a shared row block: [d][row ^ (d & 31)] fp32
+constexpr int kMaxRanges = 128;
+constexpr int kMaxTok = 264;                     // query tokens a row group of 256 rows can touch (+ slack)
+constexpr float kRescaleSlack = 8.f;             // log2 units
+static_assert(4 * kPartBytes <= kMainBytes, "partials must fit the tile buffers");
+static_assert(kNKB == 2, "the shared-block schedule assumes two key blocks per tile");
+
+struct AttnKParams {
+  const __bf16* q;
+  const __bf16* k_new;
+  const __bf16* v_new;
+  __bf16* out;
+  const void* k_cache;
+  const void* v_cache;
+  const float* k_scale;
+  const float* v_scale;
+  const int* block_table;
+  const int* q_start_loc;
+  const int* range_ptr;
+  const int* range_start;
+  const int* range_len;
+  const int* slot_table;  // [n_req, slot_stride]: cache slot of every visible prefix key; last entry = key count
+  long slot_stride;
+  const uint8_t* mask;
+  float* ws_o;
+  float* ws_lse;
+  long q_stride, kn_stride, vn_stride, o_stride;
+  long cache_page_stride, cache_token_stride, cache_head_stride;
+  long mask_stride;
+  long n_tokens;
+  int n_pages;
+  int bt_stride;
+  int scale_page_stride, scale_head_stride;
+  int n_req, Hq, Hkv, G;
+  int page_shift;
+  int max_ctx_len;
+  int max_ranges;
+  int mask_mode;
+  int J;
+  int row_tiles;
+  // work decomposition: the tiles of all columns (request, KV head, row group) form one line of
+  // n_cols * t_lin positions that is cut into spans of `span` tiles, one per workgroup
+  int t_lin;       // positions per column (>= the largest tile count of a column)
+  int span;        // tiles per workgroup
+  int n_lin;       // length of the line
+  int max_pieces;  // partial results per row in the workspace
+  // head == 0: one line over all columns (n_lin = columns * t_lin).  head > 0: the row_tiles columns of
+  // one (request, KV head), which read the same K/V tiles, form a set of wg_set workgroups: the first
+  // row_tiles of them take the first `head` tiles of one column each, side by side over the same
+  // tiles, which they share in L2; the others cut the line of the columns' remaining t_lin - head
+  // tiles (n_lin = row_tiles * (t_lin - head) positions) into spans.
+  int head;
+  int wg_set;
+  int max_q_len;
+  float scale_log2;  // sm_scale * log2(e)
+};
+
+// combine lane l with lane l ^ 32: v_permlane32_swap exchanges the upper half of its first
+// operand with the lower half of its second, so swapping a value with itself yields
+// {lower half in every lane, upper half in every lane}
+__device__ __forceinline__ float half_swap_max(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_swap_sum(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// position swizzle of the 16 chunks of a row: rotate the low 4 row bits left by one
+__device__ __forceinline__ int swz(int row) {
+  const int r = row & 15;
+  return ((r & 7) << 1) | (r >> 3);
+}
+
+// 8 e4m3 values (two dwords) * scale -> 8 bf16 (four dwords)
+__device__ __forceinline__ uint4 dequant_fp8x8(uint32_t lo, uint32_t hi, float scale) {
+  f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false);
+  f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8(lo, true);
+  f32x2 c = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
+  f32x2 d = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+  uint4 r;
+  r.x = pack_bf16x2(a[0] * scale, a[1] * scale);
+  r.y = pack_bf16x2(b[0] * scale, b[1] * scale);
+  r.z = pack_bf16x2(c[0] * scale, c[1] * scale);
+  r.w = pack_bf16x2(d[0] * scale, d[1] * scale);
+  return r;
+}
+
+// LDS operand reads of the MFMA loops are issued and awaited by hand.  The compiler would make
+// every LDS read wait for the direct-to-LDS copies of the next tile that are in flight (it
+// cannot tell that they go to the other buffer), which serialises copy and compute.  The asm
+// reads are invisible to its wait-count bookkeeping, so each consumer waits explicitly:
+// lds_wait<N>(x) blocks until at most N younger LDS operations are outstanding and ties the
+// wait to the registers x that the operation filled.
+template <int OFF>
+__device__ __forceinline__ void lds_read_b128(bf16x8& dst, unsigned addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int OFF>
+__device__ __forceinline__ void lds_read_tr16_b64(s16x4& dst, unsigned addr) {
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int N, typename T>
+__device__ __forceinline__ void lds_wait(T& x) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N) : "memory");
+}
+// the same, and also a fence for three values of the vector pipeline: work that produces them
+// stays before this point, work that consumes them after it (pins the interleaving of softmax
+// arithmetic with the MFMAs, which the compiler would otherwise gather in one place)
+// `keep` is only named as an input: it holds the fragment the MFMA of the step before is still
+// reading, and naming it here keeps the register allocator from handing those registers to the
+// vector instructions in between (a write to a source of a running MFMA stalls the wave until
+// the MFMA has finished, which would serialise the two pipelines).
+template <int N, typename T>
+__device__ __forceinline__ void lds_wait_pin(T& x, float& a, float& b, float& c, const T& keep) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(x), "+v"(a), "+v"(b), "+v"(c) : "n"(N), "v"(keep) : "memory");
+}
+template <int N, typename T>
+__device__ __forceinline__ void lds_wait2(T& x, T& y) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N) : "memory");
+}
+
+}  // namespace pdllm
