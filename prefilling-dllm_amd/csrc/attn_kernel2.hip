@@ -1,13 +1,23 @@
 // Sparse-prefix attention for gfx950, wide form: a workgroup of 4 wavefronts owns 256 rows, every wave two
 // 32-row blocks.  Each K fragment (and each V^T fragment) a wave reads from LDS feeds two MFMAs, one per row
-// block, which halves the LDS operand traffic per MFMA against one block per wave -- at one block per wave
-// every MFMA needs a fresh 1 KB fragment, which is the whole LDS bandwidth of a compute unit.  The price is the
-// register file: two sets of Q fragments, accumulators and scores need more than 256 registers per lane, so a
-// compute unit holds one such workgroup (one wave per SIMD, up to 512 registers) and all overlap of matrix,
-// vector and LDS work is arranged inside the wave: while the vector unit turns the scores of tile t into
-// probabilities, the matrix unit computes the scores of tile t + 1.
+// block, which halves the LDS operand traffic per MFMA against one block per wave (there every MFMA needs a
+// fresh 1 KB fragment, which is the whole LDS bandwidth of a compute unit).  The price is the register file:
+// two sets of Q fragments and accumulators need more than 256 registers per lane, so a compute unit holds one
+// such workgroup (one wave per SIMD, up to 512 registers) and all overlap of matrix, vector and LDS work is
+// arranged inside the wave.
 //
-// Same work decomposition, data layout in LDS, slot table, masks, partial results and epilogue as
+// A wave alone on its SIMD issues one instruction per issue slot, so every instruction of the softmax costs
+// time that no other wave fills.  The loop therefore runs as a pipeline over blocks of 32 keys in which the
+// matrix and the vector work are spread evenly: the step of block k computes the scores of block k + 1 (16
+// MFMAs), turns the scores of block k into probabilities (32 values per lane) and multiplies the
+// probabilities of block k - 1 with V (16 MFMAs) -- one exponential between any two MFMAs.  The running
+// maximum of a row is advanced when a block exceeds it by more than 2^8; the accumulators are rescaled at the
+// end of the step, when the MFMAs that still belong to the old maximum have been issued.
+//
+// K and V tiles (64 keys) live in two rings of three LDS buffers: a step reads K one block ahead and V one
+// block behind, and the copies of the tiles after the next land while a whole tile is computed.
+//
+// Same work decomposition, swizzled LDS tile layout, slot table, masks, partial results and output path as
 // attn_fwd_kernel (attn_kernel.hip); bf16 caches only.  Replaces the same reference code:
 // layers/attention/attention_v4.py:336-397, layers/attention/ops/prefix_prefill.py:25-230.
 
@@ -17,14 +27,62 @@
 
 namespace pdllm {
 
-template <int N, typename T>
-__device__ __forceinline__ void lds_wait_pin2(T& x, float& a0, float& a1, float& b0, float& b1, float& pa, float& pb,
-                                              const T& keep) {
-  asm volatile("s_waitcnt lgkmcnt(%7)"
-               : "+v"(x), "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1), "+v"(pa), "+v"(pb)
-               : "n"(N), "v"(keep)
-               : "memory");
+namespace {
+
+constexpr int kRing = 3;                          // tiles per ring
+constexpr int kVRing = kRing * kTileBytes;        // byte offset of the V ring behind the K ring
+constexpr int kWideLds = 2 * kRing * kTileBytes;  // 98304
+
+// LDS reads of one step, in the order they are issued: K fragment q (one ds_read_b128) feeds slot 2q, V^T
+// fragment v (two ds_read_b64_tr_b16) feeds slot 2v + 1; fragments 0 and 1 of each kind are issued before the
+// first slot, fragment f + 2 right after fragment f has been consumed.  Returns how many younger reads may
+// still be outstanding when the fragment of `slot` is needed (the operand of s_waitcnt lgkmcnt).
+constexpr int sched_wait(bool qk, bool pv, int slot) {
+  int issued = 0;
+  int k_pos[8] = {0, 0, 0, 0, 0, 0, 0, 0}, v_pos[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int f = 0; f < 2; ++f) {
+    if (qk) { k_pos[f] = issued; issued += 1; }
+    if (pv) { issued += 2; v_pos[f] = issued - 1; }
+  }
+  for (int s = 0; s < 16; ++s) {
+    const int f = s >> 1;
+    const bool is_k = (s & 1) == 0;
+    if (is_k ? !qk : !pv) continue;
+    if (s == slot) return issued - 1 - (is_k ? k_pos[f] : v_pos[f]);
+    if (f + 2 < 8) {
+      if (is_k) { k_pos[f + 2] = issued; issued += 1; }
+      else { issued += 2; v_pos[f + 2] = issued - 1; }
+    }
+  }
+  return 0;
 }
+
+template <int N, typename T>
+__device__ __forceinline__ void lds_wait_k(T& x) {
+  static_assert(N >= 0 && N <= 7, "unexpected LDS queue depth");
+  if constexpr (N == 0) lds_wait<0>(x);
+  else if constexpr (N == 1) lds_wait<1>(x);
+  else if constexpr (N == 2) lds_wait<2>(x);
+  else if constexpr (N == 3) lds_wait<3>(x);
+  else if constexpr (N == 4) lds_wait<4>(x);
+  else if constexpr (N == 5) lds_wait<5>(x);
+  else if constexpr (N == 6) lds_wait<6>(x);
+  else lds_wait<7>(x);
+}
+template <int N, typename T>
+__device__ __forceinline__ void lds_wait_v(T& x, T& y) {
+  static_assert(N >= 0 && N <= 7, "unexpected LDS queue depth");
+  if constexpr (N == 0) lds_wait2<0>(x, y);
+  else if constexpr (N == 1) lds_wait2<1>(x, y);
+  else if constexpr (N == 2) lds_wait2<2>(x, y);
+  else if constexpr (N == 3) lds_wait2<3>(x, y);
+  else if constexpr (N == 4) lds_wait2<4>(x, y);
+  else if constexpr (N == 5) lds_wait2<5>(x, y);
+  else if constexpr (N == 6) lds_wait2<6>(x, y);
+  else lds_wait2<7>(x, y);
+}
+
+}  // namespace
 
 #ifdef ATTN_PROBE
 __device__ unsigned long long g_probe[8 * 1024];
@@ -35,17 +93,17 @@ __device__ unsigned long long g_probe[8 * 1024];
 
 template <bool BUF>
 __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) {
+  constexpr int NW = 4;                // wavefronts per workgroup
+  constexpr int NB = 2;                // row blocks per wave
+  constexpr int J = NW * NB;           // row blocks per workgroup
+  constexpr int kDmaGroups = 16 / NW;  // a tile is 16 groups of 4 rows; a wave copies this many of them
 #ifdef ATTN_PROBE
   unsigned long long pr_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   unsigned long long pr_last = __builtin_amdgcn_s_memtime();
   const unsigned long long pr_start = pr_last;
 #endif
-  constexpr int NW = 4;                // wavefronts per workgroup
-  constexpr int NB = 2;                // row blocks per wave
-  constexpr int J = NW * NB;           // row blocks per workgroup
-  constexpr int kDmaGroups = 16 / NW;  // a tile is 16 groups of 4 rows; a wave copies this many of them
 
-  __shared__ __attribute__((aligned(1024))) char lds[kMainBytes];
+  __shared__ __attribute__((aligned(1024))) char lds[kWideLds];
   // dynamic part: the dense-mask bit rows [2][kMaxTok][kNKB] of an active tile (only with PDLLM_MASK_DENSE)
   extern __shared__ __attribute__((aligned(16))) char dyn_lds[];
   uint32_t (*s_maskbits)[kMaxTok][kNKB] = reinterpret_cast<uint32_t (*)[kMaxTok][kNKB]>(dyn_lds);
@@ -59,24 +117,6 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
   const int G = p.G;
   const float c = p.scale_log2;
   const unsigned lds_base = (unsigned)(size_t)lds;
-
-  // LDS addresses of this lane's operand fragments in buffer 0 (K: 128-bit reads of row l32 of a key block;
-  // V: transposing 64-bit reads); they move to the other buffer after every tile
-  unsigned ka[8], va[2][4];
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks) ka[ks] = lds_base + l32 * kRowBytes + (((2 * ks + h) ^ swz(l32)) << 4);
-  {
-    const int i16 = lane & 15, g4 = l32 >> 4;
-#pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      const int keyrow = 4 * h + 8 * r + (i16 >> 2);
-#pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        const int cg = 4 * db + 2 * g4 + ((i16 & 3) >> 1);
-        va[r][db] = lds_base + keyrow * kRowBytes + ((cg ^ swz(keyrow)) << 4) + ((i16 & 1) << 3);
-      }
-    }
-  }
 
   // this workgroup's span of the tile line (see attn_fwd_kernel)
   const int wg = xcd_remap(blockIdx.x, gridDim.x);
@@ -202,26 +242,22 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
     const unsigned cache_row16 = (unsigned)((p.cache_token_stride * 2) >> 4);  // 16-byte units
     const unsigned kn_row16 = (unsigned)((p.kn_stride * 2) >> 4);
     const unsigned vn_row16 = (unsigned)((p.vn_stride * 2) >> 4);
-    int nslot[kDmaGroups];  // slots of the next K tile
-    int nsv[kDmaGroups];    // slots of the next V tile
-    auto load_slots_ctx = [&](int t) __attribute__((always_inline)) {
-#pragma unroll
-      for (int i = 0; i < kDmaGroups; ++i) nslot[i] = tbl[t * kKT + 4 * NW * i + lane_row];
-    };
-    auto load_slots_new = [&](int t) __attribute__((always_inline)) {
-#pragma unroll
-      for (int i = 0; i < kDmaGroups; ++i) nslot[i] = (t - Tc) * kKT + 4 * NW * i + lane_row;
-    };
-    auto load_slots = [&](int t) __attribute__((always_inline)) {
+    int nslot[kDmaGroups];  // slots of the next K tile to copy
+    int nsv[kDmaGroups];    // slots of the next V tile to copy
+    int nnext[kDmaGroups];  // slots of the tile after those, on their way from the slot table
+    auto load_slots = [&](int (&dst)[kDmaGroups], int t) __attribute__((always_inline)) {
       if (t < Tc) {
 #pragma unroll
-        for (int i = 0; i < kDmaGroups; ++i) nslot[i] = tbl[t * kKT + 4 * NW * i + lane_row];
+        for (int i = 0; i < kDmaGroups; ++i) dst[i] = tbl[t * kKT + 4 * NW * i + lane_row];
       } else {
-        const int a0 = (t - Tc) * kKT;
+        // padding rows copy the first row of the tile, tiles past the end of the column the last tile's rows: always
+        // a valid row (they are masked, or never read)
+        int a0 = (t - Tc) * kKT;
+        a0 = a0 < (Ta - 1) * kKT ? a0 : (Ta - 1) * kKT;
 #pragma unroll
         for (int i = 0; i < kDmaGroups; ++i) {
           const int a = a0 + 4 * NW * i + lane_row;
-          nslot[i] = a < Sa ? a : a0;  // padding rows copy the first (always valid) row; they are masked
+          dst[i] = a < Sa ? a : a0;
         }
       }
     };
@@ -242,299 +278,365 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
       }
     };
-    // src_tag: 0 = decide by the tile number, 1 = the tile comes from the cache, 2 = from the new rows
-    auto issue_k1 = [&](int t, int buf, int i, auto src_tag) __attribute__((always_inline)) {
-      constexpr int SRC = decltype(src_tag)::value;
-      const bool ctx = SRC == 1 || (SRC == 0 && t < Tc);
-      copy_row(ctx ? kc_base : kn_base, ctx ? cache_row16 : kn_row16, nslot[i],
-               lds + buf * kBufBytes + wave * 1024 + i * (NW * 1024));
+    // Copy of rows of group i of a K / V tile into ring buffer `ring` (a tile number modulo kRing).  The source of a
+    // tile (cache through its slots for prefix tiles, else the new rows) is chosen once per tile: src_k / src_v.
+    struct TileSrc { const char* base; unsigned row16; };
+    auto src_of = [&](int t, const char* cache, const char* fresh, unsigned fresh_row16) __attribute__((always_inline)) {
+      TileSrc r;
+      const bool ctx = t < Tc;
+      r.base = ctx ? cache : fresh;
+      r.row16 = ctx ? cache_row16 : fresh_row16;
+      return r;
     };
-    auto issue_v1 = [&](int t, int buf, int i, auto src_tag) __attribute__((always_inline)) {
-      constexpr int SRC = decltype(src_tag)::value;
-      const bool ctx = SRC == 1 || (SRC == 0 && t < Tc);
-      copy_row(ctx ? vc_base : vn_base, ctx ? cache_row16 : vn_row16, nsv[i],
-               lds + buf * kBufBytes + kTileBytes + wave * 1024 + i * (NW * 1024));
+    auto issue_k1 = [&](const TileSrc& src, int ring, int i) __attribute__((always_inline)) {
+      copy_row(src.base, src.row16, nslot[i], lds + ring * kTileBytes + wave * 1024 + i * (NW * 1024));
     };
-    auto rdk = [&](bf16x8& dst, int stp) __attribute__((always_inline)) {
-      if ((stp >> 3) == 0) lds_read_b128<0>(dst, ka[stp & 7]);
-      else lds_read_b128<32 * kRowBytes>(dst, ka[stp & 7]);
+    auto issue_v1 = [&](const TileSrc& src, int ring, int i) __attribute__((always_inline)) {
+      copy_row(src.base, src.row16, nsv[i], lds + kVRing + ring * kTileBytes + wave * 1024 + i * (NW * 1024));
     };
-    auto rdv = [&](s16x4& dst, int stp, int r) __attribute__((always_inline)) {
-      constexpr int base = kTileBytes;
-      const int db = stp & 3, kj = stp >> 2;
-      if (kj == 0) lds_read_tr16_b64<base>(dst, va[r][db]);
-      else if (kj == 1) lds_read_tr16_b64<base + 16 * kRowBytes>(dst, va[r][db]);
-      else if (kj == 2) lds_read_tr16_b64<base + 32 * kRowBytes>(dst, va[r][db]);
-      else lds_read_tr16_b64<base + 48 * kRowBytes>(dst, va[r][db]);
-    };
-    constexpr int PF = 3, NS = 16;  // K fragments read ahead; MFMA steps of a phase
 
     if (T0 < T1) {
       typedef __attribute__((ext_vector_type(8))) short s16x8;
-      int flip = kBufBytes;  // ka: buffer 1 -> 0 -> 1 ..., va: buffer 0 -> 1 -> 0 ...
+      // LDS addresses of this lane's operand fragments (K: 128-bit reads of row l32 of a key block; V:
+      // transposing 64-bit reads).  ka points into the ring buffer of the K tile whose blocks the next QK reads,
+      // va into that of the V tile the next PV reads; both move on by one tile in the middle of an iteration.
+      unsigned ka[8], va[2][4];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) ka[ks] = lds_base + l32 * kRowBytes + (((2 * ks + h) ^ swz(l32)) << 4);
+      {
+        const int i16 = lane & 15, g4 = l32 >> 4;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const int keyrow = 4 * h + 8 * r + (i16 >> 2);
+#pragma unroll
+          for (int db = 0; db < 4; ++db) {
+            const int cg = 4 * db + 2 * g4 + ((i16 & 3) >> 1);
+            va[r][db] = lds_base + kVRing + keyrow * kRowBytes + ((cg ^ swz(keyrow)) << 4) + ((i16 & 1) << 3);
+          }
+        }
+      }
+      int k_ring = 0;  // ring buffer ka points into
+      int v_ring = 0;  // ring buffer va points into
 
-      // One iteration: softmax of tile t (raw scores in Sc) interleaved with QK of tile t + 1, then PV of tile t.
-      // PAR = buffer of V(t); K(t+1) sits in the other buffer.  MODE 1 / 2: tiles t .. t + 3 are whole tiles of
-      // the prefix / of the active block inside this piece and tile t needs no mask for any row.
-      auto iter = [&](int t, int PAR, f32x16 (&Sc)[NB][2], auto steady_tag) __attribute__((always_inline)) {
-        constexpr int MODE = decltype(steady_tag)::value;
-        constexpr bool STEADY = MODE != 0;
-        const bool has_next = STEADY || t + 1 < T1;
-        const bool k_on = STEADY || t + 2 < T1;
-        PROBE_T(0)
-        if (!STEADY && has_next) build_mask(t + 1, PAR ^ 1);
+      // K fragment ks of key block `half` of the tile at ka; V^T fragment (16 keys kj of block `half`, columns db)
+      auto rdk = [&](bf16x8& dst, int half, int ks) __attribute__((always_inline)) {
+        if (half == 0) lds_read_b128<0>(dst, ka[ks]);
+        else lds_read_b128<32 * kRowBytes>(dst, ka[ks]);
+      };
+      auto rdv = [&](s16x4& dst, int half, int v, int r) __attribute__((always_inline)) {
+        const int db = v & 3, kj = 2 * half + (v >> 2);
+        if (kj == 0) lds_read_tr16_b64<0>(dst, va[r][db]);
+        else if (kj == 1) lds_read_tr16_b64<16 * kRowBytes>(dst, va[r][db]);
+        else if (kj == 2) lds_read_tr16_b64<32 * kRowBytes>(dst, va[r][db]);
+        else lds_read_tr16_b64<48 * kRowBytes>(dst, va[r][db]);
+      };
 
-        const bool active = !STEADY && t >= Tc;
-        const int a0 = active ? (t - Tc) * kKT : 0;
-        int nvalid = STEADY ? kKT : active ? Sa - a0 : ctx_total - t * kKT;
-        const bool generic = !STEADY && (nvalid < kKT || (active && p.mask_mode != PDLLM_MASK_FULL));
-        nvalid = nvalid < kKT ? nvalid : kKT;
-        // ---- masks, row maxima, lazy rescale (vector unit only) ----
+      f32x16 S[2][NB];        // raw scores of the block being exponentiated / of the block after it
+      uint32_t Pw[2][NB][8];  // probabilities of the block before / of this block, two bf16 per word
+#pragma unroll
+      for (int rb = 0; rb < NB; ++rb)
+#pragma unroll
+        for (int w = 0; w < 8; ++w) Pw[1][rb][w] = 0u;  // "the block before the first one": contributes nothing
+      bool pending = false;   // the accumulators still have to be rescaled by alpha[]
+      float alpha[NB] = {1.f, 1.f};
+
+      // One step of the pipeline.  E = parity of block k inside its tile (0: first 32 keys).
+      //   softmax of block k: scores S[E] -> Pw[E]          (masks: lim[rb] = visible keys of the tile, mrow)
+      //   scores of block k + 1 -> S[E ^ 1]                 (K block E ^ 1 of the tile at ka)
+      //   O += V^T P^T of block k - 1 with Pw[E ^ 1]        (V block E ^ 1 of the tile at va)
+      //   dma(f): called once in every even slot for the copies of the tiles ahead
+      // There is one form of the step: before the first block the probabilities are zero and the V tile read is the
+      // first one itself; after the last block the scores of a block that does not exist are computed from
+      // whatever the K ring holds and never used.
+      auto step = [&](auto e_tag, bool generic, const int (&lim)[NB], const uint32_t* const (&mrow)[NB],
+                      auto&& dma) __attribute__((always_inline)) {
+        constexpr int E = decltype(e_tag)::value;
+        f32x16 (&Sc)[NB] = S[E];
+        f32x16 (&Sn)[NB] = S[E ^ 1];
+        bf16x8 kf[3];
+        s16x4 vlo[2], vhi[2];
+        // ---- masks (rare), row maxima of block k, decision about the running maximum ----
         if (generic) {
 #pragma unroll
           for (int rb = 0; rb < NB; ++rb) {
-            int lim = nvalid;
-            if (active && p.mask_mode == PDLLM_MASK_CAUSAL) {
-              const int cl = srow[rb] - a0 + 1;
-              lim = cl < lim ? cl : lim;
-            }
-            int tl = srow[rb] - tq_first;
-            tl = tl < 0 ? 0 : (tl >= kMaxTok ? kMaxTok - 1 : tl);
-            const uint32_t* mrow =
-                (active && p.mask_mode == PDLLM_MASK_DENSE) ? &s_maskbits[PAR][tl][0] : nullptr;
-            if (mrow != nullptr || __builtin_amdgcn_ballot_w64(lim < kKT) != 0) {
+            if (mrow[rb] != nullptr || __builtin_amdgcn_ballot_w64(lim[rb] < kKT) != 0) {
+              const int lb = lim[rb] - 32 * E;
+              uint32_t W = lb >= 32 ? 0xffffffffu : (lb <= 0 ? 0u : ((1u << lb) - 1u));
+              if (mrow[rb] != nullptr) W &= mrow[rb][E];
+              W >>= 4 * h;
 #pragma unroll
-              for (int b = 0; b < 2; ++b) {
-                const int lb = lim - 32 * b;
-                uint32_t W = lb >= 32 ? 0xffffffffu : (lb <= 0 ? 0u : ((1u << lb) - 1u));
-                if (mrow != nullptr) W &= mrow[b];
-                W >>= 4 * h;
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                  constexpr uint32_t one = 1u;
-                  const uint32_t bit = one << (8 * (i >> 2) + (i & 3));
-                  Sc[rb][b][i] = (W & bit) ? Sc[rb][b][i] : -INFINITY;
-                }
+              for (int i = 0; i < 16; ++i) {
+                constexpr uint32_t one = 1u;
+                const uint32_t bit = one << (8 * (i >> 2) + (i & 3));
+                Sc[rb][i] = (W & bit) ? Sc[rb][i] : -INFINITY;
               }
             }
           }
         }
+        // fragments 0 and 1 of each kind
+#pragma unroll
+        for (int f = 0; f < 2; ++f) {
+          rdk(kf[f], E ^ 1, f);
+          rdv(vlo[f], E ^ 1, f, 0);
+          rdv(vhi[f], E ^ 1, f, 1);
+        }
+#pragma unroll
+        for (int rb = 0; rb < NB; ++rb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) Sn[rb][i] = 0.f;
         float mx[NB];
         bool need = false;
 #pragma unroll
         for (int rb = 0; rb < NB; ++rb) {
-          float m0 = fmaxf(Sc[rb][0][0], Sc[rb][0][1]);
+          float m0 = fmaxf(Sc[rb][0], Sc[rb][1]);
 #pragma unroll
-          for (int b = 0; b < 2; ++b)
-#pragma unroll
-            for (int i = (b == 0 ? 2 : 0); i < 16; i += 2) m0 = fmaxf(fmaxf(m0, Sc[rb][b][i]), Sc[rb][b][i + 1]);
-          mx[rb] = half_swap_max(m0) * c;  // log2 units
+          for (int i = 2; i < 16; i += 2) m0 = fmaxf(fmaxf(m0, Sc[rb][i]), Sc[rb][i + 1]);
+          mx[rb] = half_swap_max(m0) * c;  // log2 units; -inf (nothing visible) stays -inf
           need = need || mx[rb] > M[rb] + kRescaleSlack;
         }
         if (__builtin_amdgcn_ballot_w64(need) != 0) {
 #pragma unroll
           for (int rb = 0; rb < NB; ++rb) {
             const float Mn = fmaxf(M[rb], mx[rb]);
-            const float alpha = (Mn == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(M[rb] - Mn);
+            const float a = (Mn == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(M[rb] - Mn);  // M = -inf -> 0
+            alpha[rb] = a;
             M[rb] = Mn;
-            l[rb] *= alpha;
-#pragma unroll
-            for (int db = 0; db < 4; ++db) {
-#pragma unroll
-              for (int i = 0; i < 16; ++i) O[rb][db][i] *= alpha;
-              __builtin_amdgcn_sched_barrier(0);
-            }
+            l[rb] *= a;
           }
+          pending = true;
         }
-        PROBE_T(1)
-        // ---- exponentials of tile t, two per row block and step, between the MFMAs of QK(t+1) ----
         float negM[NB];
 #pragma unroll
         for (int rb = 0; rb < NB; ++rb) negM[rb] = (M[rb] == -INFINITY) ? 0.f : -M[rb];
-        f32x16 Sn[NB][2];
-#pragma unroll
-        for (int rb = 0; rb < NB; ++rb)
-#pragma unroll
-          for (int b = 0; b < 2; ++b)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) Sn[rb][b][i] = 0.f;
-        bf16x8 P[NB][2][2];
         const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
         float psum[NB] = {0.f, 0.f};
-        auto exp_pair = [&](int rb, int stp) __attribute__((always_inline)) {
-          const int b = stp >> 3, i = 2 * (stp & 7);
-          const bf16x2 pr = {(__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(Sc[rb][b][i], c, negM[rb])),
-                             (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(Sc[rb][b][i + 1], c, negM[rb]))};
-          psum[rb] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum[rb], false);
-          P[rb][b][i >> 3][i & 7] = pr[0];
-          P[rb][b][i >> 3][(i & 7) + 1] = pr[1];
+        // B operand of the second MFMA: 8 probabilities (keys 16 j .. 16 j + 15 of the block, this lane's half)
+        auto p_frag = [&](int e, int rb, int j) __attribute__((always_inline)) {
+          const uint4 w = {Pw[e][rb][4 * j], Pw[e][rb][4 * j + 1], Pw[e][rb][4 * j + 2], Pw[e][rb][4 * j + 3]};
+          return __builtin_bit_cast(bf16x8, w);
         };
-        if (has_next) {
-          bf16x8 kf[PF];
+        auto exp2s = [&](float e, int rb) __attribute__((always_inline)) {
+          return __builtin_amdgcn_exp2f(__builtin_fmaf(e, c, negM[rb]));
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- 16 slots of two MFMAs each.  A wave alone on its SIMD issues in order, and the matrix unit takes a new
+        // MFMA every 32 clocks: the second MFMA of a slot would hold up everything behind it, so each half of a slot
+        // is one MFMA followed by the arithmetic of one probability (pair pr = s of the block: row block s / 8,
+        // scores 2 (s % 8) and + 1).  The scores and the intermediate results pass through (empty) asm statements
+        // of their half: that keeps the arithmetic there -- the instruction selector would otherwise gather all of
+        // it in one place.
 #pragma unroll
-          for (int i = 0; i < PF; ++i) rdk(kf[i], i);
-          bf16x8 used = kf[0];  // fragment of the MFMAs issued in the step before
+        for (int s = 0; s < 16; ++s) {
+          const int f = s >> 1;
+          const int prb = s >> 3, pi = 2 * (s & 7);
+          float e0 = Sc[prb][pi], e1 = Sc[prb][pi + 1];
+          bf16x8 frag;
+          if ((s & 1) == 0) {
+            // wait for K fragment f
+            if (s == 0) lds_wait_k<sched_wait(true, true, 0)>(kf[f % 3]);
+            else if (s == 2) lds_wait_k<sched_wait(true, true, 2)>(kf[f % 3]);
+            else if (s == 4) lds_wait_k<sched_wait(true, true, 4)>(kf[f % 3]);
+            else if (s == 6) lds_wait_k<sched_wait(true, true, 6)>(kf[f % 3]);
+            else if (s == 8) lds_wait_k<sched_wait(true, true, 8)>(kf[f % 3]);
+            else if (s == 10) lds_wait_k<sched_wait(true, true, 10)>(kf[f % 3]);
+            else if (s == 12) lds_wait_k<sched_wait(true, true, 12)>(kf[f % 3]);
+            else lds_wait_k<sched_wait(true, true, 14)>(kf[f % 3]);
+            frag = kf[f % 3];
+          } else {
+            if (s == 1) lds_wait_v<sched_wait(true, true, 1)>(vlo[f & 1], vhi[f & 1]);
+            else if (s == 3) lds_wait_v<sched_wait(true, true, 3)>(vlo[f & 1], vhi[f & 1]);
+            else if (s == 5) lds_wait_v<sched_wait(true, true, 5)>(vlo[f & 1], vhi[f & 1]);
+            else if (s == 7) lds_wait_v<sched_wait(true, true, 7)>(vlo[f & 1], vhi[f & 1]);
+            else if (s == 9) lds_wait_v<sched_wait(true, true, 9)>(vlo[f & 1], vhi[f & 1]);
+            else if (s == 11) lds_wait_v<sched_wait(true, true, 11)>(vlo[f & 1], vhi[f & 1]);
+            else if (s == 13) lds_wait_v<sched_wait(true, true, 13)>(vlo[f & 1], vhi[f & 1]);
+            else lds_wait_v<sched_wait(true, true, 15)>(vlo[f & 1], vhi[f & 1]);
+            const s16x4 a = vlo[f & 1], b2 = vhi[f & 1];
+            const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
+            frag = __builtin_bit_cast(bf16x8, both);
+          }
+          // ---- first half: MFMA of row block 0, first probability ----
+          asm volatile("" : "+v"(e0), "+v"(psum[prb]));
+          if ((s & 1) == 0) Sn[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, Q[0][f], Sn[0], 0, 0, 0);
+          else O[0][f & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, p_frag(E ^ 1, 0, f >> 2), O[0][f & 3], 0, 0, 0);
+          float x0 = exp2s(e0, prb);
           __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int stp = 0; stp < NS; ++stp) {
-            const int kb = stp >> 3, ks = stp & 7, e = 2 * ks;
-            {
-              float a0s = Sc[0][kb][e], a1s = Sc[0][kb][e + 1], b0s = Sc[1][kb][e], b1s = Sc[1][kb][e + 1];
-              const int young = NS - 1 - stp < PF - 1 ? NS - 1 - stp : PF - 1;
-              if (young == 2) lds_wait_pin2<2>(kf[stp % PF], a0s, a1s, b0s, b1s, psum[0], psum[1], used);
-              else if (young == 1) lds_wait_pin2<1>(kf[stp % PF], a0s, a1s, b0s, b1s, psum[0], psum[1], used);
-              else lds_wait_pin2<0>(kf[stp % PF], a0s, a1s, b0s, b1s, psum[0], psum[1], used);
-              used = kf[stp % PF];
-              Sc[0][kb][e] = a0s; Sc[0][kb][e + 1] = a1s; Sc[1][kb][e] = b0s; Sc[1][kb][e + 1] = b1s;
-            }
-            if (ks == 7) {
-              // the block's exponentials are all issued: its registers take the finished scores
-              exp_pair(0, stp);
-              exp_pair(1, stp);
-              Sc[0][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], Q[0][7], Sn[0][kb], 0, 0, 0);
-              Sc[1][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], Q[1][7], Sn[1][kb], 0, 0, 0);
-            } else {
-              Sn[0][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], Q[0][ks], Sn[0][kb], 0, 0, 0);
-              Sn[1][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], Q[1][ks], Sn[1][kb], 0, 0, 0);
-              exp_pair(0, stp);
-              exp_pair(1, stp);
-            }
-            if (stp + PF < NS) rdk(kf[stp % PF], stp + PF);
-            if ((stp & 1) == 1 && (ks >> 1) < kDmaGroups) {
-              if (stp < 8) issue_v1(t + 1, PAR ^ 1, ks >> 1, steady_tag);
-              else if (k_on) issue_k1(t + 2, PAR, ks >> 1, steady_tag);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+          // ---- second half: MFMA of row block 1, second probability, pack, row sum; next fragment ----
+          asm volatile("" : "+v"(e1), "+v"(x0));
+          if ((s & 1) == 0) {
+            Sn[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, Q[1][f], Sn[1], 0, 0, 0);
+            if (f + 2 < 8) rdk(kf[(f + 2) % 3], E ^ 1, f + 2);
+            dma(f);
+          } else {
+            O[1][f & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, p_frag(E ^ 1, 1, f >> 2), O[1][f & 3], 0, 0, 0);
+            if (f + 2 < 8) { rdv(vlo[f & 1], E ^ 1, f + 2, 0); rdv(vhi[f & 1], E ^ 1, f + 2, 1); }
           }
-#pragma unroll
-          for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
-          if (MODE == 1) load_slots_ctx(t + 3);
-          else if (MODE == 2) load_slots_new(t + 3);
-          else if (t + 3 < T1) load_slots(t + 3);
-        } else {
-#pragma unroll
-          for (int stp = 0; stp < NS; ++stp) {
-            exp_pair(0, stp);
-            exp_pair(1, stp);
-          }
+          const float x1 = exp2s(e1, prb);
+          const bf16x2 pv2 = {(__bf16)x0, (__bf16)x1};
+          psum[prb] = __builtin_amdgcn_fdot2_f32_bf16(pv2, ones, psum[prb], false);
+          Pw[E][prb][s & 7] = __builtin_bit_cast(uint32_t, pv2);
+          __builtin_amdgcn_sched_barrier(0);
         }
+        asm volatile("" : "+v"(psum[0]), "+v"(psum[1]));
         l[0] += psum[0];
         l[1] += psum[1];
-        __builtin_amdgcn_sched_barrier(0);
-        PROBE_T(2)
-        // ---- PV of tile t: every V^T fragment feeds both row blocks ----
-        {
-          s16x4 lo[2], hi[2];
-          rdv(lo[0], 0, 0); rdv(hi[0], 0, 1);
-          rdv(lo[1], 1, 0); rdv(hi[1], 1, 1);
-          __builtin_amdgcn_sched_barrier(0);
+        // the accumulators follow the running maximum once every MFMA of the old one has been issued
+        if (pending) {
 #pragma unroll
-          for (int stp = 0; stp < NS; ++stp) {
-            const int db = stp & 3, kj = stp >> 2;
-            if (stp + 1 < NS) lds_wait2<2>(lo[stp & 1], hi[stp & 1]);
-            else lds_wait2<0>(lo[stp & 1], hi[stp & 1]);
-            const s16x4 a = lo[stp & 1], b2 = hi[stp & 1];
-            const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
-            const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
-            O[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P[0][kj >> 1][kj & 1], O[0][db], 0, 0, 0);
-            O[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P[1][kj >> 1][kj & 1], O[1][db], 0, 0, 0);
-            if (stp + 2 < NS) { rdv(lo[stp & 1], stp + 2, 0); rdv(hi[stp & 1], stp + 2, 1); }
-            __builtin_amdgcn_sched_barrier(0);
-          }
+          for (int rb = 0; rb < NB; ++rb)
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+#pragma unroll
+              for (int i = 0; i < 16; ++i) O[rb][db][i] *= alpha[rb];
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          pending = false;
         }
-        PROBE_T(3)
-        // the next tile reads the other buffers
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) ka[ks] -= flip;
-#pragma unroll
-        for (int r = 0; r < 2; ++r)
-#pragma unroll
-          for (int db = 0; db < 4; ++db) va[r][db] += flip;
-        flip = -flip;
-#ifndef EXP_NOWAIT
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): K(t+2), V(t+1) and the slots have landed
-#endif
-        PROBE_T(4)
-        __syncthreads();
-        PROBE_T(5)
       };
 
-      // ---- prologue: K(T0), V(T0); then K(T0+1) while QK(T0) runs unpipelined ----
-      f32x16 SX[NB][2];
-      load_slots(T0);
+      // ---- prologue: K(T0), V(T0), K(T0+1); scores of the first block ----
+      load_slots(nslot, T0);
 #pragma unroll
       for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
+      {
+        const TileSrc sk = src_of(T0, kc_base, kn_base, kn_row16), sv = src_of(T0, vc_base, vn_base, vn_row16);
 #pragma unroll
-      for (int i = 0; i < kDmaGroups; ++i) issue_k1(T0, 0, i, std::integral_constant<int, 0>{});
+        for (int i = 0; i < kDmaGroups; ++i) issue_k1(sk, 0, i);
 #pragma unroll
-      for (int i = 0; i < kDmaGroups; ++i) issue_v1(T0, 0, i, std::integral_constant<int, 0>{});
-      if (T0 + 1 < T1) load_slots(T0 + 1);
+        for (int i = 0; i < kDmaGroups; ++i) issue_v1(sv, 0, i);
+      }
+      {
+        // (like the copies inside the loop, issued whether or not the piece has a second tile: the slots loaded for a
+        // tile and the source chosen for it always belong together)
+        load_slots(nslot, T0 + 1);
+        const TileSrc sk = src_of(T0 + 1, kc_base, kn_base, kn_row16);
+#pragma unroll
+        for (int i = 0; i < kDmaGroups; ++i) issue_k1(sk, 1, i);
+      }
+#pragma unroll
+      for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];  // slots of tile T0 + 1 for its V copy
+      load_slots(nslot, T0 + 2);
       build_mask(T0, 0);
       __builtin_amdgcn_s_waitcnt(0x0F70);
       __syncthreads();
-      if (T0 + 1 < T1) {
-#pragma unroll
-        for (int i = 0; i < kDmaGroups; ++i) issue_k1(T0 + 1, 1, i, std::integral_constant<int, 0>{});
-      }
-#pragma unroll
-      for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
-      if (T0 + 2 < T1) load_slots(T0 + 2);
-#pragma unroll
-      for (int rb = 0; rb < NB; ++rb)
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) SX[rb][b][i] = 0.f;
       {
-        bf16x8 kf[PF];
+        // scores of block 0 (unpipelined)
 #pragma unroll
-        for (int i = 0; i < PF; ++i) rdk(kf[i], i);
+        for (int rb = 0; rb < NB; ++rb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) S[0][rb][i] = 0.f;
+        bf16x8 kf[3];
+        rdk(kf[0], 0, 0);
+        rdk(kf[1], 0, 1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int stp = 0; stp < NS; ++stp) {
-          const int young = NS - 1 - stp < PF - 1 ? NS - 1 - stp : PF - 1;
-          if (young == 2) lds_wait<2>(kf[stp % PF]);
-          else if (young == 1) lds_wait<1>(kf[stp % PF]);
-          else lds_wait<0>(kf[stp % PF]);
-          SX[0][stp >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], Q[0][stp & 7], SX[0][stp >> 3], 0, 0, 0);
-          SX[1][stp >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], Q[1][stp & 7], SX[1][stp >> 3], 0, 0, 0);
-          if (stp + PF < NS) rdk(kf[stp % PF], stp + PF);
+        for (int f = 0; f < 8; ++f) {
+          if (f + 2 < 8) { rdk(kf[(f + 2) % 3], 0, f + 2); lds_wait<2>(kf[f % 3]); }
+          else if (f + 1 < 8) lds_wait<1>(kf[f % 3]);
+          else lds_wait<0>(kf[f % 3]);
+          S[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[f % 3], Q[0][f], S[0][0], 0, 0, 0);
+          S[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[f % 3], Q[1][f], S[0][1], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-      // from here on ka reads K(t+1) in buffer 1 and va reads V(t) in buffer 0
+      // ---- the tiles of the piece: one loop, one form of the iteration (two steps) ----
+      for (int t = T0; t < T1; ++t) {
+        const int par = (t - T0) & 1;
+        const bool has_next = t + 1 < T1;
+        PROBE_T(0)
+        // the slots of tile t + 3 are fetched first, while no copy is in flight
+        load_slots(nnext, t + 3);
+        if (has_next) build_mask(t + 1, par ^ 1);
+        const bool active = t >= Tc;
+        const int a0 = active ? (t - Tc) * kKT : 0;
+        int nvalid = active ? Sa - a0 : ctx_total - t * kKT;
+        const bool generic = nvalid < kKT || (active && p.mask_mode != PDLLM_MASK_FULL);
+        nvalid = nvalid < kKT ? nvalid : kKT;
+        int lim[NB] = {kKT, kKT};
+        const uint32_t* mrow[NB] = {nullptr, nullptr};
+        if (generic) {
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) ka[ks] += kBufBytes;
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      __syncthreads();
+          for (int rb = 0; rb < NB; ++rb) {
+            lim[rb] = nvalid;
+            if (active && p.mask_mode == PDLLM_MASK_CAUSAL) {
+              const int cl = srow[rb] - a0 + 1;
+              lim[rb] = cl < lim[rb] ? cl : lim[rb];
+            }
+            int tl = srow[rb] - tq_first;
+            tl = tl < 0 ? 0 : (tl >= kMaxTok ? kMaxTok - 1 : tl);
+            if (active && p.mask_mode == PDLLM_MASK_DENSE) mrow[rb] = &s_maskbits[par][tl][0];
+          }
+        }
+        // ring buffers: K(t) and V(t) sit in buffer (t - T0) % 3 (= k_ring here), K(t+1) in the next one; the copy
+        // of V(t+1) goes into the next one, that of K(t+2) into the one after
+        const int ring1 = k_ring + 1 >= kRing ? k_ring + 1 - kRing : k_ring + 1;
+        const int ring2 = ring1 + 1 >= kRing ? ring1 + 1 - kRing : ring1 + 1;
+        // The copies are issued whether or not the piece has a tile t + 1 / t + 2: their ring buffers are free, their
+        // slots name valid rows, and what lands there is never read (cheaper than a branch around every instruction).
+        const TileSrc src_v = src_of(t + 1, vc_base, vn_base, vn_row16);
+        const TileSrc src_k = src_of(t + 2, kc_base, kn_base, kn_row16);
+        auto dma_a = [&](int f) __attribute__((always_inline)) {
+          if (f < kDmaGroups) issue_v1(src_v, ring1, f);
+          else issue_k1(src_k, ring2, f - kDmaGroups);
+        };
+        auto no_dma = [&](int) __attribute__((always_inline)) {};
+        // step of the tile's first block: QK of its second block (same K tile), PV of the last block of tile t - 1
+        // (for the first tile: zero probabilities against the first V tile itself)
+        step(std::integral_constant<int, 0>{}, generic, lim, mrow, dma_a);
+        PROBE_T(1)
+        // K: on to tile t + 1; V: on to tile t (in the first iteration va is there already)
+        {
+          const int kn = k_ring + 1 == kRing ? 0 : k_ring + 1;
+          const int dk = (kn - k_ring) * kTileBytes;
+          k_ring = kn;
+#pragma unroll
+          for (int ks = 0; ks < 8; ++ks) ka[ks] += dk;
+          if (t > T0) {
+            const int vn = v_ring + 1 == kRing ? 0 : v_ring + 1;
+            const int dv = (vn - v_ring) * kTileBytes;
+            v_ring = vn;
+#pragma unroll
+            for (int r = 0; r < 2; ++r)
+#pragma unroll
+              for (int db = 0; db < 4; ++db) va[r][db] += dv;
+          }
+        }
+        // step of the tile's second block: QK of the first block of tile t + 1, PV of the tile's first block
+        step(std::integral_constant<int, 1>{}, generic, lim, mrow, no_dma);
+        PROBE_T(2)
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): K(t+2), V(t+1) and the slots have landed
+#pragma unroll
+        for (int i = 0; i < kDmaGroups; ++i) { nsv[i] = nslot[i]; nslot[i] = nnext[i]; }
+        PROBE_T(3)
+        __syncthreads();
+        PROBE_T(4)
+      }
+      // ---- the last block still has to be multiplied with V (second block of tile T1 - 1, at va) ----
       {
-        using Generic = std::integral_constant<int, 0>;
-        const int whole_ctx = ctx_total / kKT;  // tiles of the prefix without a ragged end
-        const int ctx_end = (T1 < whole_ctx ? T1 : whole_ctx) - 3;
-        // active tiles that are whole and visible to every row of this row group
-        int open_tiles = Sa / kKT;
-        if (p.mask_mode == PDLLM_MASK_CAUSAL) open_tiles = (tq_first + 1) / kKT < open_tiles ? (tq_first + 1) / kKT : open_tiles;
-        if (p.mask_mode == PDLLM_MASK_DENSE) open_tiles = 0;
-        int new_end = Tc + Sa / kKT - 3;
-        new_end = new_end < T1 - 3 ? new_end : T1 - 3;
-        new_end = new_end < Tc + open_tiles ? new_end : Tc + open_tiles;
-        int t = T0;
-        for (; t < ctx_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 1>{});
-        for (; t < T1 && t < Tc; ++t) iter(t, (t - T0) & 1, SX, Generic{});
-        for (; t < new_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 2>{});
-        for (; t < T1; ++t) iter(t, (t - T0) & 1, SX, Generic{});
+        s16x4 vlo[2], vhi[2];
+        rdv(vlo[0], 1, 0, 0); rdv(vhi[0], 1, 0, 1);
+        rdv(vlo[1], 1, 1, 0); rdv(vhi[1], 1, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int f = 0; f < 8; ++f) {
+          if (f + 1 < 8) lds_wait2<2>(vlo[f & 1], vhi[f & 1]);
+          else lds_wait2<0>(vlo[f & 1], vhi[f & 1]);
+          const s16x4 a = vlo[f & 1], b2 = vhi[f & 1];
+          const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
+          const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
+          const int db = f & 3, j = f >> 2;
+          const uint4 w0 = {Pw[1][0][4 * j], Pw[1][0][4 * j + 1], Pw[1][0][4 * j + 2], Pw[1][0][4 * j + 3]};
+          const uint4 w1 = {Pw[1][1][4 * j], Pw[1][1][4 * j + 1], Pw[1][1][4 * j + 2], Pw[1][1][4 * j + 3]};
+          O[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, __builtin_bit_cast(bf16x8, w0), O[0][db], 0, 0, 0);
+          O[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, __builtin_bit_cast(bf16x8, w1), O[1][db], 0, 0, 0);
+          if (f + 2 < 8) { rdv(vlo[f & 1], 1, f + 2, 0); rdv(vhi[f & 1], 1, f + 2, 1); }
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
-      // leave ka / va pointing at buffer 0 for the next piece
-      if (flip > 0) {
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) ka[ks] -= kBufBytes;
-      } else {
-#pragma unroll
-        for (int r = 0; r < 2; ++r)
-#pragma unroll
-          for (int db = 0; db < 4; ++db) va[r][db] -= kBufBytes;
-      }
+      // the output strips below reuse the K ring; every wave has left the tile loop (barrier of the last
+      // iteration) and the last V reads above go to the V ring
     }
+    PROBE_T(5)
 
     // ---- epilogue ----
     auto emit = [&](int rix, int db, const f32x16& o, float mfin, float lfin) __attribute__((always_inline)) {
@@ -551,8 +653,8 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
       }
       if (db == 0 && he == 0) p.ws_lse[R] = lfin > 0.f ? mfin + __log2f(lfin) : -INFINITY;  // log2 domain
     };
-    // rows of an uncut column go through an 8 KB strip of the (now free) tile buffers per wave, 64 columns at a
-    // time, so that 8 lanes store the 128 contiguous bytes of a row; partial rows are stored directly
+    // rows of an uncut column go through an 8 KB strip of the (now free) K ring per wave, 64 columns at a time,
+    // so that 8 lanes store the 128 contiguous bytes of a row; partial rows are stored directly
     auto emit_block = [&](int rix, const f32x16 (&Ob)[4], float mfin, float lfin) __attribute__((always_inline)) {
       if (!whole) {
 #pragma unroll
@@ -606,13 +708,13 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     }
+    PROBE_T(6)
   }  // pieces
 #ifdef ATTN_PROBE
-  PROBE_T(6)
   if ((threadIdx.x & 63) == 0 && blockIdx.x < 128) {
     unsigned long long* o = g_probe + (blockIdx.x * 4 + (threadIdx.x >> 6)) * 8;
     for (int i = 0; i < 7; ++i) o[i] = pr_acc[i];
-    o[7] = pr_last - pr_start;
+    o[7] = __builtin_amdgcn_s_memtime() - pr_start;
   }
 #endif
 }
