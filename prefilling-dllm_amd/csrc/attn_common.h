@@ -87,10 +87,15 @@ __device__ __forceinline__ float half_swap_sum(float x) {
   const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
-// position swizzle of the 16 chunks of a row: rotate the low 4 row bits left by one
+// Position swizzle of the 16 chunks (16 bytes each) of a 256-byte row: chunk c of row r sits at c ^ swz(r).  Any
+// bijection of the low four row bits keeps the 128-bit K reads (16 consecutive rows, one chunk) and the copies
+// (whole rows) free of bank conflicts.  The transposing 64-bit V reads touch, per group of 32 lanes, four rows
+// (row bits 0-1) and four neighbouring chunks of each (chunk bits 0-1): row bits 0-1 therefore go to chunk bits
+// 2-3, so that the four rows use four different quarters of the 64 banks.  (With the row bits merely rotated the
+// rows collided in pairs and every V read took two passes: measured 2x on the LDS read rate.)
 __device__ __forceinline__ int swz(int row) {
   const int r = row & 15;
-  return ((r & 7) << 1) | (r >> 3);
+  return ((r & 3) << 2) | (((r >> 2) & 1) << 1) | (r >> 3);
 }
 
 // 8 e4m3 values (two dwords) * scale -> 8 bf16 (four dwords)
