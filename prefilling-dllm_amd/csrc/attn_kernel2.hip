@@ -1,18 +1,24 @@
-// Sparse-prefix attention for gfx950, wide form: a workgroup of 4 wavefronts owns 256 rows, every wave two
-// 32-row blocks.  Each K fragment (and each V^T fragment) a wave reads from LDS feeds two MFMAs, one per row
-// block, which halves the LDS operand traffic per MFMA against one block per wave (there every MFMA needs a
-// fresh 1 KB fragment, which is the whole LDS bandwidth of a compute unit).  The price is the register file:
-// two sets of Q fragments and accumulators need more than 256 registers per lane, so a compute unit holds one
-// such workgroup (one wave per SIMD, up to 512 registers) and all overlap of matrix, vector and LDS work is
-// arranged inside the wave.
+// Sparse-prefix attention for gfx950, wide form: a workgroup owns 256 rows and runs the softmax as a pipeline
+// over blocks of 32 keys.  Two shapes of the workgroup are written here:
 //
-// A wave alone on its SIMD issues one instruction per issue slot, so every instruction of the softmax costs
-// time that no other wave fills.  The loop therefore runs as a pipeline over blocks of 32 keys in which the
-// matrix and the vector work are spread evenly: the step of block k computes the scores of block k + 1 (16
-// MFMAs), turns the scores of block k into probabilities (32 values per lane) and multiplies the
-// probabilities of block k - 1 with V (16 MFMAs) -- one exponential between any two MFMAs.  The running
-// maximum of a row is advanced when a block exceeds it by more than 2^8; the accumulators are rescaled at the
-// end of the step, when the MFMAs that still belong to the old maximum have been issued.
+//   NW = 8, NB = 1   eight wavefronts, one 32-row block each (two waves per SIMD, at most 256 registers).
+//                    This is the shape that is launched.
+//   NW = 4, NB = 2   four wavefronts, two 32-row blocks each: every K fragment (and V^T fragment) a wave reads
+//                    from LDS feeds two MFMAs, which halves the LDS operand traffic per MFMA.  It needs more
+//                    than 256 registers per lane, so a compute unit holds one wave per SIMD, and a wave alone
+//                    on its SIMD issues one instruction every 4-8 clocks whatever the instruction is: measured
+//                    on an MI355X, 32 MFMAs with the softmax arithmetic of 32 keys between them take ~1450
+//                    clocks from one wave and ~2150-2600 clocks from each of two waves sharing a SIMD (that
+//                    is 64 MFMAs), and the whole kernel came out 10-20 % slower than NW = 8 on every shape
+//                    tried (165 vs 142 us at 8 x 256 query rows over 4096 keys, 749 vs 659 us at 8 x 1024).
+//                    It is kept as a compile-time option of the same code, not instantiated.
+//
+// The loop runs as a pipeline over blocks of 32 keys in which the matrix and the vector work are spread
+// evenly: the step of block k computes the scores of block k + 1 (8 MFMAs per row block), turns the scores of
+// block k into probabilities (16 values per lane and row block) and multiplies the probabilities of block
+// k - 1 with V (8 MFMAs per row block) -- one exponential between any two MFMAs.  The running maximum of a row
+// is advanced when a block exceeds it by more than 2^8; the accumulators are rescaled at the end of the step,
+// when the MFMAs that still belong to the old maximum have been issued.
 //
 // K and V tiles (64 keys) live in two rings of three LDS buffers: a step reads K one block ahead and V one
 // block behind, and the copies of the tiles after the next land while a whole tile is computed.
@@ -84,24 +90,11 @@ __device__ __forceinline__ void lds_wait_v(T& x, T& y) {
 
 }  // namespace
 
-#ifdef ATTN_PROBE
-__device__ unsigned long long g_probe[8 * 1024];
-#define PROBE_T(i) { const unsigned long long now_ = __builtin_amdgcn_s_memtime(); pr_acc[i] += now_ - pr_last; pr_last = now_; }
-#else
-#define PROBE_T(i)
-#endif
-
-template <bool BUF>
-__global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) {
-  constexpr int NW = 4;                // wavefronts per workgroup
-  constexpr int NB = 2;                // row blocks per wave
+template <int NW, int NB, bool BUF>  // wavefronts per workgroup, row blocks per wave
+__global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams p) {
+  static_assert((NW == 4 && NB == 2) || (NW == 8 && NB == 1), "256 rows per workgroup");
   constexpr int J = NW * NB;           // row blocks per workgroup
   constexpr int kDmaGroups = 16 / NW;  // a tile is 16 groups of 4 rows; a wave copies this many of them
-#ifdef ATTN_PROBE
-  unsigned long long pr_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  unsigned long long pr_last = __builtin_amdgcn_s_memtime();
-  const unsigned long long pr_start = pr_last;
-#endif
 
   __shared__ __attribute__((aligned(1024))) char lds[kWideLds];
   // dynamic part: the dense-mask bit rows [2][kMaxTok][kNKB] of an active tile (only with PDLLM_MASK_DENSE)
@@ -338,7 +331,9 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
 #pragma unroll
         for (int w = 0; w < 8; ++w) Pw[1][rb][w] = 0u;  // "the block before the first one": contributes nothing
       bool pending = false;   // the accumulators still have to be rescaled by alpha[]
-      float alpha[NB] = {1.f, 1.f};
+      float alpha[NB];
+#pragma unroll
+      for (int rb = 0; rb < NB; ++rb) alpha[rb] = 1.f;
 
       // One step of the pipeline.  E = parity of block k inside its tile (0: first 32 keys).
       //   softmax of block k: scores S[E] -> Pw[E]          (masks: lim[rb] = visible keys of the tile, mrow)
@@ -409,7 +404,9 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
 #pragma unroll
         for (int rb = 0; rb < NB; ++rb) negM[rb] = (M[rb] == -INFINITY) ? 0.f : -M[rb];
         const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
-        float psum[NB] = {0.f, 0.f};
+        float psum[NB];
+#pragma unroll
+        for (int rb = 0; rb < NB; ++rb) psum[rb] = 0.f;
         // B operand of the second MFMA: 8 probabilities (keys 16 j .. 16 j + 15 of the block, this lane's half)
         auto p_frag = [&](int e, int rb, int j) __attribute__((always_inline)) {
           const uint4 w = {Pw[e][rb][4 * j], Pw[e][rb][4 * j + 1], Pw[e][rb][4 * j + 2], Pw[e][rb][4 * j + 3]};
@@ -425,11 +422,10 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
         // scores 2 (s % 8) and + 1).  The scores and the intermediate results pass through (empty) asm statements
         // of their half: that keeps the arithmetic there -- the instruction selector would otherwise gather all of
         // it in one place.
+        float xprev = 0.f;  // NB == 1: the first probability of a pair, kept for one slot
 #pragma unroll
         for (int s = 0; s < 16; ++s) {
           const int f = s >> 1;
-          const int prb = s >> 3, pi = 2 * (s & 7);
-          float e0 = Sc[prb][pi], e1 = Sc[prb][pi + 1];
           bf16x8 frag;
           if ((s & 1) == 0) {
             // wait for K fragment f
@@ -455,31 +451,55 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
             const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
             frag = __builtin_bit_cast(bf16x8, both);
           }
-          // ---- first half: MFMA of row block 0, first probability ----
-          asm volatile("" : "+v"(e0), "+v"(psum[prb]));
-          if ((s & 1) == 0) Sn[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, Q[0][f], Sn[0], 0, 0, 0);
-          else O[0][f & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, p_frag(E ^ 1, 0, f >> 2), O[0][f & 3], 0, 0, 0);
-          float x0 = exp2s(e0, prb);
-          __builtin_amdgcn_sched_barrier(0);
-          // ---- second half: MFMA of row block 1, second probability, pack, row sum; next fragment ----
-          asm volatile("" : "+v"(e1), "+v"(x0));
-          if ((s & 1) == 0) {
-            Sn[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, Q[1][f], Sn[1], 0, 0, 0);
-            if (f + 2 < 8) rdk(kf[(f + 2) % 3], E ^ 1, f + 2);
-            dma(f);
+          if constexpr (NB == 2) {
+            const int prb = s >> 3, pi = 2 * (s & 7);
+            float e0 = Sc[prb][pi], e1 = Sc[prb][pi + 1];
+            // ---- first half: MFMA of row block 0, first probability ----
+            asm volatile("" : "+v"(e0), "+v"(psum[prb]));
+            if ((s & 1) == 0) Sn[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, Q[0][f], Sn[0], 0, 0, 0);
+            else O[0][f & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, p_frag(E ^ 1, 0, f >> 2), O[0][f & 3], 0, 0, 0);
+            float x0 = exp2s(e0, prb);
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- second half: MFMA of row block 1, second probability, pack, row sum; next fragment ----
+            asm volatile("" : "+v"(e1), "+v"(x0));
+            if ((s & 1) == 0) {
+              Sn[NB - 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, Q[NB - 1][f], Sn[NB - 1], 0, 0, 0);
+              if (f + 2 < 8) rdk(kf[(f + 2) % 3], E ^ 1, f + 2);
+              dma(f);
+            } else {
+              O[NB - 1][f & 3] =
+                  __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, p_frag(E ^ 1, NB - 1, f >> 2), O[NB - 1][f & 3], 0, 0, 0);
+              if (f + 2 < 8) { rdv(vlo[f & 1], E ^ 1, f + 2, 0); rdv(vhi[f & 1], E ^ 1, f + 2, 1); }
+            }
+            const float x1 = exp2s(e1, prb);
+            const bf16x2 pv2 = {(__bf16)x0, (__bf16)x1};
+            psum[prb] = __builtin_amdgcn_fdot2_f32_bf16(pv2, ones, psum[prb], false);
+            Pw[E][prb][s & 7] = __builtin_bit_cast(uint32_t, pv2);
           } else {
-            O[1][f & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, p_frag(E ^ 1, 1, f >> 2), O[1][f & 3], 0, 0, 0);
-            if (f + 2 < 8) { rdv(vlo[f & 1], E ^ 1, f + 2, 0); rdv(vhi[f & 1], E ^ 1, f + 2, 1); }
+            // one row block per wave: one MFMA and one probability per slot, a pair is packed in every odd slot
+            float e = Sc[0][s];
+            asm volatile("" : "+v"(e), "+v"(psum[0]), "+v"(xprev));
+            if ((s & 1) == 0) {
+              Sn[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, Q[0][f], Sn[0], 0, 0, 0);
+              if (f + 2 < 8) rdk(kf[(f + 2) % 3], E ^ 1, f + 2);
+              dma(f);
+              xprev = exp2s(e, 0);
+            } else {
+              O[0][f & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, p_frag(E ^ 1, 0, f >> 2), O[0][f & 3], 0, 0, 0);
+              if (f + 2 < 8) { rdv(vlo[f & 1], E ^ 1, f + 2, 0); rdv(vhi[f & 1], E ^ 1, f + 2, 1); }
+              const float x1 = exp2s(e, 0);
+              const bf16x2 pv2 = {(__bf16)xprev, (__bf16)x1};
+              psum[0] = __builtin_amdgcn_fdot2_f32_bf16(pv2, ones, psum[0], false);
+              Pw[E][0][s >> 1] = __builtin_bit_cast(uint32_t, pv2);
+            }
           }
-          const float x1 = exp2s(e1, prb);
-          const bf16x2 pv2 = {(__bf16)x0, (__bf16)x1};
-          psum[prb] = __builtin_amdgcn_fdot2_f32_bf16(pv2, ones, psum[prb], false);
-          Pw[E][prb][s & 7] = __builtin_bit_cast(uint32_t, pv2);
           __builtin_amdgcn_sched_barrier(0);
         }
-        asm volatile("" : "+v"(psum[0]), "+v"(psum[1]));
-        l[0] += psum[0];
-        l[1] += psum[1];
+#pragma unroll
+        for (int rb = 0; rb < NB; ++rb) {
+          asm volatile("" : "+v"(psum[rb]));
+          l[rb] += psum[rb];
+        }
         // the accumulators follow the running maximum once every MFMA of the old one has been issued
         if (pending) {
 #pragma unroll
@@ -534,8 +554,9 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
           if (f + 2 < 8) { rdk(kf[(f + 2) % 3], 0, f + 2); lds_wait<2>(kf[f % 3]); }
           else if (f + 1 < 8) lds_wait<1>(kf[f % 3]);
           else lds_wait<0>(kf[f % 3]);
-          S[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[f % 3], Q[0][f], S[0][0], 0, 0, 0);
-          S[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[f % 3], Q[1][f], S[0][1], 0, 0, 0);
+#pragma unroll
+          for (int rb = 0; rb < NB; ++rb)
+            S[0][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[f % 3], Q[rb][f], S[0][rb], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -543,7 +564,6 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
       for (int t = T0; t < T1; ++t) {
         const int par = (t - T0) & 1;
         const bool has_next = t + 1 < T1;
-        PROBE_T(0)
         // the slots of tile t + 3 are fetched first, while no copy is in flight
         load_slots(nnext, t + 3);
         if (has_next) build_mask(t + 1, par ^ 1);
@@ -552,8 +572,10 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
         int nvalid = active ? Sa - a0 : ctx_total - t * kKT;
         const bool generic = nvalid < kKT || (active && p.mask_mode != PDLLM_MASK_FULL);
         nvalid = nvalid < kKT ? nvalid : kKT;
-        int lim[NB] = {kKT, kKT};
-        const uint32_t* mrow[NB] = {nullptr, nullptr};
+        int lim[NB];
+        const uint32_t* mrow[NB];
+#pragma unroll
+        for (int rb = 0; rb < NB; ++rb) { lim[rb] = kKT; mrow[rb] = nullptr; }
         if (generic) {
 #pragma unroll
           for (int rb = 0; rb < NB; ++rb) {
@@ -577,13 +599,12 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
         const TileSrc src_k = src_of(t + 2, kc_base, kn_base, kn_row16);
         auto dma_a = [&](int f) __attribute__((always_inline)) {
           if (f < kDmaGroups) issue_v1(src_v, ring1, f);
-          else issue_k1(src_k, ring2, f - kDmaGroups);
+          else if (f < 2 * kDmaGroups) issue_k1(src_k, ring2, f - kDmaGroups);
         };
         auto no_dma = [&](int) __attribute__((always_inline)) {};
         // step of the tile's first block: QK of its second block (same K tile), PV of the last block of tile t - 1
         // (for the first tile: zero probabilities against the first V tile itself)
         step(std::integral_constant<int, 0>{}, generic, lim, mrow, dma_a);
-        PROBE_T(1)
         // K: on to tile t + 1; V: on to tile t (in the first iteration va is there already)
         {
           const int kn = k_ring + 1 == kRing ? 0 : k_ring + 1;
@@ -603,13 +624,10 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
         }
         // step of the tile's second block: QK of the first block of tile t + 1, PV of the tile's first block
         step(std::integral_constant<int, 1>{}, generic, lim, mrow, no_dma);
-        PROBE_T(2)
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): K(t+2), V(t+1) and the slots have landed
 #pragma unroll
         for (int i = 0; i < kDmaGroups; ++i) { nsv[i] = nslot[i]; nslot[i] = nnext[i]; }
-        PROBE_T(3)
         __syncthreads();
-        PROBE_T(4)
       }
       // ---- the last block still has to be multiplied with V (second block of tile T1 - 1, at va) ----
       {
@@ -625,18 +643,19 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
           const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
           const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
           const int db = f & 3, j = f >> 2;
-          const uint4 w0 = {Pw[1][0][4 * j], Pw[1][0][4 * j + 1], Pw[1][0][4 * j + 2], Pw[1][0][4 * j + 3]};
-          const uint4 w1 = {Pw[1][1][4 * j], Pw[1][1][4 * j + 1], Pw[1][1][4 * j + 2], Pw[1][1][4 * j + 3]};
-          O[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, __builtin_bit_cast(bf16x8, w0), O[0][db], 0, 0, 0);
-          O[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, __builtin_bit_cast(bf16x8, w1), O[1][db], 0, 0, 0);
+#pragma unroll
+          for (int rb = 0; rb < NB; ++rb) {
+            const uint4 w = {Pw[1][rb][4 * j], Pw[1][rb][4 * j + 1], Pw[1][rb][4 * j + 2], Pw[1][rb][4 * j + 3]};
+            O[rb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, __builtin_bit_cast(bf16x8, w), O[rb][db], 0, 0, 0);
+          }
           if (f + 2 < 8) { rdv(vlo[f & 1], 1, f + 2, 0); rdv(vhi[f & 1], 1, f + 2, 1); }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
       // the output strips below reuse the K ring; every wave has left the tile loop (barrier of the last
-      // iteration) and the last V reads above go to the V ring
+      // iteration) and the last V reads above go to the V ring -- which the strips of eight waves reach into
+      if constexpr (NW * 8192 > kVRing) __syncthreads();
     }
-    PROBE_T(5)
 
     // ---- epilogue ----
     auto emit = [&](int rix, int db, const f32x16& o, float mfin, float lfin) __attribute__((always_inline)) {
@@ -708,27 +727,14 @@ __global__ __launch_bounds__(256, 1) void attn_fwd2_kernel(const AttnKParams p) 
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     }
-    PROBE_T(6)
   }  // pieces
-#ifdef ATTN_PROBE
-  if ((threadIdx.x & 63) == 0 && blockIdx.x < 128) {
-    unsigned long long* o = g_probe + (blockIdx.x * 4 + (threadIdx.x >> 6)) * 8;
-    for (int i = 0; i < 7; ++i) o[i] = pr_acc[i];
-    o[7] = __builtin_amdgcn_s_memtime() - pr_start;
-  }
-#endif
 }
 
 int launch_attn_fwd2(const AttnKParams& p, int grid, int dyn_lds, bool buf, hipStream_t stream) {
-  if (buf) hipLaunchKernelGGL((attn_fwd2_kernel<true>), dim3((unsigned)grid), dim3(256), dyn_lds, stream, p);
-  else hipLaunchKernelGGL((attn_fwd2_kernel<false>), dim3((unsigned)grid), dim3(256), dyn_lds, stream, p);
+  if (buf) hipLaunchKernelGGL((attn_fwd2_kernel<8, 1, true>), dim3((unsigned)grid), dim3(512), dyn_lds, stream, p);
+  else hipLaunchKernelGGL((attn_fwd2_kernel<8, 1, false>), dim3((unsigned)grid), dim3(512), dyn_lds, stream, p);
   return launch_status();
 }
 
 }  // namespace pdllm
 
-#ifdef ATTN_PROBE
-extern "C" int pdllm_debug_probe(unsigned long long* host_out) {
-  return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(pdllm::g_probe), sizeof(unsigned long long) * 8 * 1024) == hipSuccess ? 0 : -1;
-}
-#endif
