@@ -319,7 +319,14 @@ int pdllm_kv_copy_pages(const void* src_cache, void* dst_cache, const int32_t* s
  * n_seqs blocks of block_len rows of bf16 logits [n_seqs*block_len, vocab]:
  * row i of block b reads logits row (b*block_len + i - shift) where shift = 1 uses
  * last_logit[b] (or the block's own row 0 when last_logit == NULL) for i = 0;
- * confidence = max softmax probability in fp32, token = first index of the maximum. */
+ * confidence = max softmax probability in fp32, token = first index of the maximum.
+ * Accuracy: the token is exact (integer comparison of the bf16 logits, first index on ties).  The confidence is
+ * 1 / sum_j exp(x_j - max) with the sum taken in fp32 over fixed per-lane and per-split partial sums, an order
+ * that differs from torch.softmax's; the two agree to within 5e-5 absolute (the bound the parity tests hold, on
+ * vocabularies up to 152064).  Everything that compares the confidence with a threshold (pdllm_threshold_unmask,
+ * pdllm_denoise_unmask*) therefore decides exactly as the reference whenever the reference's confidence is
+ * further than 5e-5 from the threshold; inside that band either decision can come out.  The most confident
+ * position of a block is always transferred, so a block never stalls on such a tie. */
 int pdllm_conf_argmax(const void* logits, int64_t logits_stride, const void* last_logit,
                       int64_t last_logit_stride, int64_t n_seqs, int64_t block_len, int64_t vocab,
                       int32_t shift, void* workspace, int64_t workspace_bytes, float* conf_out,

@@ -28,6 +28,8 @@ How each function is pinned (tests/test_oracle_*.py):
   vote keep set : numpy bincount + stable argsort, and the invariants of the definition (first token of a
       chunk and tokens outside the chunks survive, min(capacity, length) per chunk, no dropped token
       outvotes a kept one)
+  draft rounds : a hand-computed 3-round trace on a 5-token vocabulary (which position wins each round, ties)
+  keep-list assembly : a hand-listed example with a leading gap, adjacent chunks and a tail
   anchor corrections : hand-listed anchor / window tables for the three directions, stride 1 with a zero window
       reproduces the dense result, an unchanged prompt gives a zero delta, the selection modes reduce to the plain
       mode for selection == dense
@@ -612,3 +614,54 @@ def threshold_unmask(block_ids: torch.Tensor, confidence: torch.Tensor, sampled:
             transfer[idx] = True
     block_ids[transfer] = sampled[transfer]
     return block_ids, transfer
+
+
+def partial_draft_rounds(logits_of, prompt_ids: Sequence[int], max_new_tokens: int, partial_rounds: int,
+                         mask_token_id: int) -> Tuple[List[int], List[bool]]:
+    """ENG:1013-1059 with the model forward abstracted: logits_of(ids list) -> [len(ids), vocab] tensor.
+    First the token at block position 0 is confirmed, then one masked position per round: the one whose
+    (shifted) confidence is the highest, first on ties."""
+    draft_len = int(max_new_tokens or 0)
+    if draft_len <= 0:
+        return [], []
+    prompt_ids = [int(x) for x in prompt_ids]
+    block_ids = [int(mask_token_id)] * draft_len
+    confirmed = [False] * draft_len
+    n = len(prompt_ids)
+    shifted = shift_logits(logits_of(prompt_ids + block_ids))
+    _, first = sample_tokens(shifted[n:n + 1])
+    block_ids[0] = int(first[0])
+    confirmed[0] = True
+    for _ in range(max(0, int(partial_rounds or 0))):
+        mask_positions = [i for i, t in enumerate(block_ids) if t == mask_token_id]
+        if not mask_positions:
+            break
+        shifted = shift_logits(logits_of(prompt_ids + block_ids))
+        conf, tok = sample_tokens(shifted[n:n + draft_len][mask_positions])
+        best = int(torch.argmax(conf))
+        block_ids[mask_positions[best]] = int(tok[best])
+        confirmed[mask_positions[best]] = True
+    return block_ids, confirmed
+
+
+def assemble_global_keep_indices(layer_chunk_keeps, chunk_spans, full_prompt_len: int, num_kv_heads: int):
+    """ENG:1524-1546, head by head: gaps between the processed chunks are kept whole, each chunk contributes its
+    (already global) keep list.  layer_chunk_keeps[layer][chunk] = [Hkv][kept] ints; returns [layer][head][pos]."""
+    out = []
+    for parts in layer_chunk_keeps:
+        if not parts:
+            out.append([list(range(full_prompt_len)) for _ in range(num_kv_heads)])
+            continue
+        heads = []
+        for h in range(len(parts[0])):
+            pieces, cursor = [], 0
+            for (start, end), keep in zip(chunk_spans, parts):
+                if start > cursor:
+                    pieces += list(range(cursor, start))
+                pieces += [int(x) for x in keep[h]]
+                cursor = end
+            if cursor < full_prompt_len:
+                pieces += list(range(cursor, full_prompt_len))
+            heads.append(pieces)
+        out.append(heads)
+    return out

@@ -6,15 +6,13 @@ error behaviour follow the reference methods (cited per function; ENG = fastdllm
 from __future__ import annotations
 
 import math
-import threading
-from collections import deque
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
-import numpy as np
 import torch
 
 from . import ops
+from .page_pool import PageAllocator, PagePool, PrefixPageAllocator, _CachedPrefix  # noqa: F401  (re-exported)
 
 PAGE_SIZE = ops.PAGE_SIZE
 
@@ -60,88 +58,6 @@ class DreamKVSnapshot:
     k_by_layer: List[torch.Tensor]
     v_by_layer: List[torch.Tensor]
     last_context_logit: Optional[torch.Tensor] = None
-
-
-@dataclass
-class _CachedPrefix:
-    prompt_hash: int
-    page_ids: List[int]
-    prompt_len: int
-    last_context_logit: torch.Tensor
-    ref_count: int = 1
-
-
-class PrefixPageAllocator:
-    """Free-list page allocator with per-page refcounts and hash-keyed prefix sharing (ENG:88-167).
-    Host-side integers only; it stays Python as in the reference."""
-
-    def __init__(self, num_pages: int, page_size: int):
-        self.num_pages = num_pages
-        self.page_size = page_size
-        self.free_pages: deque = deque(range(num_pages))
-        self.page_ref_count: List[int] = [0] * num_pages
-        self.hash_to_prefix: Dict[int, _CachedPrefix] = {}
-        self._lock = threading.RLock()
-
-    @staticmethod
-    def compute_prompt_hash(prompt_ids: List[int]) -> int:
-        import xxhash
-        h = xxhash.xxh64()
-        h.update(np.array(prompt_ids, dtype=np.int64).tobytes())
-        return h.intdigest()
-
-    @property
-    def num_free_pages(self) -> int:
-        with self._lock:
-            return len(self.free_pages)
-
-    def allocate_pages(self, n: int) -> List[int]:
-        with self._lock:
-            if n > len(self.free_pages):
-                raise RuntimeError(f"Cannot allocate {n} pages, only {len(self.free_pages)} free")
-            pages = [self.free_pages.popleft() for _ in range(n)]
-            for p in pages:
-                self.page_ref_count[p] = 1
-            return pages
-
-    def ref_pages(self, pages: List[int]) -> None:
-        with self._lock:
-            for p in pages:
-                self.page_ref_count[p] += 1
-
-    def release_pages(self, pages: List[int]) -> None:
-        with self._lock:
-            for p in pages:
-                self.page_ref_count[p] -= 1
-                if self.page_ref_count[p] == 0:
-                    self.free_pages.append(p)
-
-    def lookup_prefix(self, prompt_ids: List[int]) -> Optional[_CachedPrefix]:
-        with self._lock:
-            return self.hash_to_prefix.get(self.compute_prompt_hash(prompt_ids))
-
-    def register_prefix(self, prompt_ids, page_ids, prompt_len, last_context_logit) -> _CachedPrefix:
-        with self._lock:
-            h = self.compute_prompt_hash(prompt_ids)
-            entry = _CachedPrefix(prompt_hash=h, page_ids=list(page_ids), prompt_len=prompt_len,
-                                  last_context_logit=last_context_logit.detach(), ref_count=0)
-            self.hash_to_prefix[h] = entry
-            return entry
-
-    def release_prefix(self, prompt_ids: List[int]) -> None:
-        with self._lock:
-            entry = self.hash_to_prefix.get(self.compute_prompt_hash(prompt_ids))
-            if entry is not None:
-                entry.ref_count -= 1
-
-    def evict_one(self) -> bool:
-        with self._lock:
-            for h, entry in list(self.hash_to_prefix.items()):
-                if entry.ref_count <= 0:
-                    self.release_pages(entry.page_ids)
-                    del self.hash_to_prefix[h]
-                    return True
-            return False
 
 
 # ------------------------------------------------------------------------------------------
@@ -348,7 +264,7 @@ def snapshot_pd_record_kv(kv_cache: torch.Tensor, record: DreamPrefillRecord, *,
                            last_context_logit=None if ll is None else ll.to(device))
 
 
-def _allocate_record_pages(allocator: PrefixPageAllocator, prompt_len: int, decode_len: int,
+def _allocate_record_pages(allocator: PageAllocator, prompt_len: int, decode_len: int,
                            page_size: int) -> Tuple[List[int], List[int]]:
     """Pages for a record on the decode side: evict unreferenced cached prefixes until both lists fit
     (ENG:746-751), then take the prompt pages and the block pages."""
@@ -371,7 +287,7 @@ def _decode_side_record(source: DreamPrefillRecord, prompt_page_ids: List[int], 
         kv_mode=source.kv_mode)
 
 
-def make_pd_record_from_kv_snapshot(kv_cache: torch.Tensor, allocator: PrefixPageAllocator,
+def make_pd_record_from_kv_snapshot(kv_cache: torch.Tensor, allocator: PageAllocator,
                                     source: DreamPrefillRecord, snapshot: DreamKVSnapshot, *,
                                     page_size: int = PAGE_SIZE) -> DreamPrefillRecord:
     """make_pd_record_from_kv_snapshot (ENG:728-781): allocate local pages, load the snapshot into them
@@ -392,7 +308,7 @@ def make_pd_record_from_kv_snapshot(kv_cache: torch.Tensor, allocator: PrefixPag
 
 
 def make_pd_record_from_remote_cache(src_kv_cache: torch.Tensor, dst_kv_cache: torch.Tensor,
-                                     allocator: PrefixPageAllocator, source: DreamPrefillRecord, *,
+                                     allocator: PageAllocator, source: DreamPrefillRecord, *,
                                      page_size: int = PAGE_SIZE) -> DreamPrefillRecord:
     """make_pd_record_from_remote_engine (ENG:800-881) for two caches on this GPU: the prompt KV moves
     page by page, all layers in one launch, instead of one gather and one indexed write per layer."""
@@ -414,7 +330,7 @@ def make_pd_record_from_remote_cache(src_kv_cache: torch.Tensor, dst_kv_cache: t
     return _decode_side_record(source, prompt_pages, block_pages, ll)
 
 
-def release_pd_record(allocator: PrefixPageAllocator, record: DreamPrefillRecord) -> None:
+def release_pd_record(allocator: PageAllocator, record: DreamPrefillRecord) -> None:
     """release_pd_record (ENG:2192-2198): block pages always go back, prompt pages when the record owns
     them, and a shared prefix loses one reference."""
     allocator.release_pages(record.block_page_ids)
@@ -514,3 +430,104 @@ def denoise_unmask_step(logits: torch.Tensor, block_ids: torch.Tensor, *, mask_t
     _, _, transfer, left = ops.denoise_unmask(logits, block_ids, mask_token_id, threshold, shift=shift,
                                               last_logit=last_context_logit)
     return transfer, left
+
+
+# ------------------------------------------------------------------------------------------
+# draft rounds for chunk selection (ENG:1013-1059)
+# ------------------------------------------------------------------------------------------
+
+def partial_draft_round(logits: torch.Tensor, block_ids: torch.Tensor, *, prompt_len: int, mask_token_id: int,
+                        first: bool = False) -> torch.Tensor:
+    """One round of generate_partial_draft_rounds_for_selection (ENG:1043-1059) on the device, no host sync.
+
+    logits [prompt_len + draft_len, vocab] bf16 is the model output for prompt + block, block_ids [draft_len] or
+    [1, draft_len] int64 is updated in place.  A round confirms exactly one position: the still-masked position
+    whose shifted logits are the most confident (first one on ties) receives its argmax token -- the unmask step
+    with a threshold no confidence reaches.  first=True is the opening move of the reference (ENG:1034-1036): position
+    0 is confirmed whatever its confidence.  Returns the bool transfer mask of the round, shaped like block_ids.
+
+    The shift needs no copy: shifted row prompt_len + i is logits row prompt_len + i - 1 (ENG:1647-1656), so the
+    block's shifted rows are the slice starting at prompt_len - 1; with an empty prompt row 0 stands for itself."""
+    ids = block_ids.view(1, -1)
+    draft_len = ids.shape[1]
+    if logits.dim() != 2 or logits.shape[0] != prompt_len + draft_len:
+        raise ValueError("logits must be [prompt_len + draft_len, vocab]")
+    if prompt_len > 0:
+        rows, shift = logits[prompt_len - 1:prompt_len - 1 + draft_len], False
+    else:
+        rows, shift = logits, True
+    if first:
+        rows, ids = rows[:1], ids[:, :1]
+        if not bool(ids.is_contiguous()):
+            raise ValueError("block_ids must be contiguous")
+    _, _, transfer, _ = ops.denoise_unmask(rows, ids, mask_token_id, 2.0, shift=shift)
+    if first:
+        full = torch.zeros(draft_len, dtype=torch.bool, device=logits.device)
+        full[:1] = transfer.view(-1)
+        transfer = full
+    return transfer.view(block_ids.shape)
+
+
+def generate_partial_draft_rounds_for_selection(forward_logits, prompt_ids: Sequence[int], *, max_new_tokens: int,
+                                                partial_rounds: int, mask_token_id: int,
+                                                device=None) -> Tuple[List[int], List[bool]]:
+    """generate_partial_draft_rounds_for_selection (ENG:1013-1059) around a caller-supplied model forward:
+    forward_logits(token_ids int64 [prompt_len + draft_len]) -> logits [prompt_len + draft_len, vocab] bf16 stands
+    for _forward_prefill_for_selection with a full mask.  The block stays on the device between rounds; the only
+    host transfers are the two result lists at the end (the reference reads one scalar per round to find the masked
+    positions).  A round after the last mask is gone changes nothing, as the reference's early exit."""
+    draft_len = int(max_new_tokens or 0)
+    if draft_len <= 0:
+        return [], []
+    prompt = torch.as_tensor([int(x) for x in prompt_ids], dtype=torch.int64, device=device)
+    dev = prompt.device
+    block = torch.full((draft_len,), int(mask_token_id), dtype=torch.int64, device=dev)
+    confirmed = torch.zeros(draft_len, dtype=torch.bool, device=dev)
+    n = int(prompt.numel())
+    for r in range(1 + max(0, int(partial_rounds or 0))):
+        logits = forward_logits(torch.cat([prompt, block]))
+        confirmed |= partial_draft_round(logits, block, prompt_len=n, mask_token_id=mask_token_id, first=(r == 0))
+    return block.tolist(), confirmed.tolist()
+
+
+# ------------------------------------------------------------------------------------------
+# per-chunk keep lists -> global keep lists (ENG:1524-1546)
+# ------------------------------------------------------------------------------------------
+
+def assemble_global_keep_indices(layer_chunk_keeps: Sequence[Sequence[torch.Tensor]],
+                                 chunk_spans: Sequence[Tuple[int, int]], full_prompt_len: int, num_kv_heads: int,
+                                 as_lists: bool = True):
+    """Global keep lists per layer and KV head from the keep lists of the evicted chunks (ENG:1524-1546).
+
+    layer_chunk_keeps[layer][c] is int64 [Hkv, kept_c]: the positions kept of chunk c, already global (the engine
+    adds the chunk start, ENG:1514); chunk_spans[c] = (start, end) in the order the chunks were processed.
+    Everything outside the spans is kept by every head: the result of a head is, span after span, the gap in front
+    of the span (cursor .. start) followed by the span's kept positions, then the tail up to full_prompt_len.  A
+    layer without keep lists keeps every position.  Returns List[layer][head][position] (as_lists, the reference's
+    form, the input of normalize_per_head_keep_indices / compact_prompt_cache_per_layer_per_head) or a list of
+    int64 tensors [Hkv, n] on the device of the keep lists."""
+    spans = [(int(s[0]), int(s[1])) if not isinstance(s, dict) else (int(s["start"]), int(s["end"]))
+             for s in chunk_spans]
+    out = []
+    for parts in layer_chunk_keeps:
+        parts = list(parts)
+        if not parts:
+            t = torch.arange(full_prompt_len, dtype=torch.int64).unsqueeze(0).repeat(int(num_kv_heads), 1)
+            out.append(t.tolist() if as_lists else t)
+            continue
+        if len(parts) != len(spans):
+            raise ValueError("one keep tensor per chunk span expected")
+        dev, heads = parts[0].device, int(parts[0].shape[0])
+        cols, cursor = [], 0
+        for (start, end), keep in zip(spans, parts):
+            if keep.dim() != 2 or int(keep.shape[0]) != heads:
+                raise ValueError("keep lists must be [Hkv, kept] with the same Hkv for every chunk")
+            if start > cursor:                      # whole rows of columns: the gap is the same for every head
+                cols.append(torch.arange(cursor, start, dtype=torch.int64, device=dev).expand(heads, -1))
+            cols.append(keep.to(device=dev, dtype=torch.int64))
+            cursor = end
+        if cursor < full_prompt_len:
+            cols.append(torch.arange(cursor, full_prompt_len, dtype=torch.int64, device=dev).expand(heads, -1))
+        t = torch.cat(cols, dim=1)
+        out.append(t.tolist() if as_lists else t)
+    return out

@@ -98,28 +98,67 @@ def test_attention_plan_is_host_only():
     assert ops.attention_plan(8, 28, 4, max_q_len=160, max_ctx_len=4096, rows_per_group=128, num_splits=2) == (128, 2)
 
 
-def test_prefix_page_allocator_semantics():
-    """fastdllm_engine.py:88-167: free-list order, refcounts, exhaustion error, hash-keyed prefix reuse."""
-    from prefilling_dllm_amd.engine_ops import PrefixPageAllocator
+def test_page_pool_semantics():
+    """What callers of the reference's allocator observe (fastdllm_engine.py:88-167): pages are handed out in the
+    order they became free, refcounts, the exhaustion error, hash-keyed prefix reuse and eviction."""
+    from prefilling_dllm_amd.page_pool import PageAllocator, PagePool, prompt_digest
+    from prefilling_dllm_amd import engine_ops
     import torch
-    a = PrefixPageAllocator(4, 256)
+    assert engine_ops.PrefixPageAllocator is PagePool
+    a = PagePool(4, 256)
+    assert isinstance(a, PageAllocator)
     p = a.allocate_pages(3)
     assert p == [0, 1, 2] and a.num_free_pages == 1
     with pytest.raises(RuntimeError, match="Cannot allocate 2 pages, only 1 free"):
         a.allocate_pages(2)
+    assert a.num_free_pages == 1                                      # all or nothing
     a.ref_pages([1])
     a.release_pages([0, 1])
     assert a.num_free_pages == 2 and a.page_ref_count[1] == 1        # page 1 still referenced
     a.release_pages([1])
     assert list(a.free_pages) == [3, 0, 1]
+    with pytest.raises(RuntimeError, match="released more often"):
+        a.release_pages([3])
     ids = [5, 6, 7]
     e = a.register_prefix(ids, [2], 3, torch.zeros(4))
     assert a.lookup_prefix(ids) is e and a.lookup_prefix([5, 6]) is None
-    assert a.compute_prompt_hash(ids) == a.compute_prompt_hash(list(ids))
+    assert a.compute_prompt_hash(ids) == prompt_digest(tuple(ids))
+    # the digest is xxh64 over the ids as little-endian int64 (known answer: the empty prompt, and one id)
+    import xxhash
+    assert prompt_digest([]) == 0xEF46DB3751D8E999
+    assert prompt_digest([1]) == xxhash.xxh64((1).to_bytes(8, "little")).intdigest()
     e.ref_count = 1
     assert not a.evict_one()
     a.release_prefix(ids)
     assert a.evict_one() and a.lookup_prefix(ids) is None and a.num_free_pages == 4
+    assert list(a.free_pages) == [3, 0, 1, 2]
+    assert a.allocate_pages(4) == [3, 0, 1, 2] and a.num_free_pages == 0 and list(a.free_pages) == []
+    a.release_pages([1])
+    assert list(a.free_pages) == [1]
+
+
+def test_record_helpers_take_any_allocator():
+    """The PD record helpers only use allocate_pages / release_pages / evict_one / num_free_pages."""
+    from prefilling_dllm_amd import engine_ops as eo
+
+    class Counting:
+        def __init__(self):
+            self.free, self.log = list(range(10)), []
+        num_free_pages = property(lambda self: len(self.free))
+        def allocate_pages(self, n):
+            out, self.free = self.free[:n], self.free[n:]
+            return out
+        def release_pages(self, pages):
+            self.log.append(list(pages)); self.free += list(pages)
+        def evict_one(self):
+            return False
+
+    a = Counting()
+    prompt, block = eo._allocate_record_pages(a, 600, 32, 256)
+    assert prompt == [0, 1, 2] and block == [3]
+    rec = eo.DreamPrefillRecord([], [], [], 600, 600, 32, prompt, block, 0, None, None, True)
+    eo.release_pd_record(a, rec)
+    assert a.log == [[3], [0, 1, 2]]
 
 
 def test_record_types_keep_the_reference_fields():
@@ -201,3 +240,33 @@ def test_anchor_params_follow_the_reference_defaults_and_clamps():
                 lo = a - (left if direction in (0, 2) else 0)
                 hi = a + (right if direction in (1, 2) else 0)
                 assert rows == list(range(max(0, lo), min(seq_len - 1, hi) + 1)), (st, seq_len, a)
+
+
+def test_assemble_global_keep_indices_against_the_oracle():
+    """engine_ops.assemble_global_keep_indices (fastdllm_engine.py:1524-1546) on random spans and keep lists."""
+    import random
+    import torch
+    from oracle import ref_ops
+    from prefilling_dllm_amd import engine_ops as eo
+    rng = random.Random(5)
+    for case in range(20):
+        L, H, n = rng.randint(1, 3), rng.randint(1, 4), rng.randint(8, 60)
+        cuts = sorted(rng.sample(range(n + 1), rng.randint(2, 6)))
+        spans = [(a, b) for a, b in zip(cuts[:-1], cuts[1:]) if rng.random() < 0.7 and b > a] or [(cuts[0], cuts[1])]
+        layers = []
+        for layer in range(L):
+            if rng.random() < 0.2:
+                layers.append([])
+                continue
+            parts = []
+            for a, b in spans:
+                k = rng.randint(1, b - a)
+                parts.append(torch.tensor([sorted(rng.sample(range(a, b), k)) for _ in range(H)], dtype=torch.int64))
+            layers.append(parts)
+        ref = ref_ops.assemble_global_keep_indices([[p.tolist() for p in parts] for parts in layers], spans, n, H)
+        got = eo.assemble_global_keep_indices(layers, spans, n, H)
+        assert got == ref, case
+        tens = eo.assemble_global_keep_indices(layers, [{"start": a, "end": b} for a, b in spans], n, H, as_lists=False)
+        assert [t.tolist() for t in tens] == ref
+    with pytest.raises(ValueError):
+        eo.assemble_global_keep_indices([[torch.zeros(2, 1, dtype=torch.int64)]], [(0, 1), (1, 2)], 4, 2)

@@ -148,7 +148,7 @@ def test_pd_handoff_snapshot_and_page_copy(dev):
     snap = eo.snapshot_pd_record_kv(src, rec, device="cpu")
     assert snap.k_by_layer[0].device.type == "cpu" and tuple(snap.k_by_layer[0].shape) == (prompt_len, Hkv, d)
     dst = torch.zeros_like(src)
-    alloc = eo.PrefixPageAllocator(n_pages, P)
+    alloc = eo.PagePool(n_pages, P)
     alloc.allocate_pages(2)                                     # pages 0, 1 are taken by someone else
     rec2 = eo.make_pd_record_from_kv_snapshot(dst, alloc, rec, snap)
     assert rec2.prompt_page_ids == [2, 3, 4] and rec2.block_page_ids == [5] and rec2.owns_prompt_pages
@@ -167,7 +167,7 @@ def test_pd_handoff_snapshot_and_page_copy(dev):
 
     # (2) cache to cache, whole pages, all layers in one launch
     dst2 = torch.zeros_like(src)
-    alloc2 = eo.PrefixPageAllocator(n_pages, P)
+    alloc2 = eo.PagePool(n_pages, P)
     alloc2.allocate_pages(4)
     rec3 = eo.make_pd_record_from_remote_cache(src, dst2, alloc2, rec)
     assert rec3.prompt_page_ids == [4, 5, 6]

@@ -263,6 +263,62 @@ def test_unmask_all_below_threshold_moves_exactly_one(dev):
     assert nb.tolist() == [99, 8, 99, 99]
 
 
+def _toy_model(vocab, seed):
+    """A deterministic stand-in for the model forward: logits row p depends on the token ids at positions <= p
+    (so confirming a token changes the later rows, as a real forward does).  bf16 logits on the CPU."""
+    gen = torch.Generator().manual_seed(seed)
+    emb = torch.randn(vocab + 1, 48, generator=gen)
+    out = torch.randn(48, vocab, generator=gen) * 0.6
+
+    def logits_of(ids):
+        ids = torch.as_tensor(ids, dtype=torch.int64).cpu()
+        x = emb[ids.clamp(max=vocab)]
+        ctx = torch.cumsum(x, 0) / torch.arange(1, len(ids) + 1).unsqueeze(1)
+        return ((x + ctx) @ out).to(torch.bfloat16)
+
+    return logits_of
+
+
+@pytest.mark.parametrize("prompt_len,draft_len,rounds", [(7, 4, 0), (7, 4, 2), (5, 6, 5), (9, 3, 8), (0, 5, 3),
+                                                         (33, 32, 12)])
+def test_partial_draft_rounds_for_selection(dev, prompt_len, draft_len, rounds):
+    """engine_ops.generate_partial_draft_rounds_for_selection against the restatement of
+    fastdllm_engine.py:1013-1059: same tokens, same confirmed positions, round by round (each round is the device
+    unmask step with a threshold no confidence reaches, position 0 first)."""
+    from prefilling_dllm_amd import engine_ops as eo
+    vocab, mask_id = 3000, 3000
+    model = _toy_model(vocab, 100 + prompt_len)
+    prompt = list(range(11, 11 + prompt_len))
+    ref_ids, ref_conf = ref_ops.partial_draft_rounds(lambda ids: model(ids).float(), prompt, draft_len, rounds, mask_id)
+    got_ids, got_conf = eo.generate_partial_draft_rounds_for_selection(
+        lambda ids: model(ids).to(dev), prompt, max_new_tokens=draft_len, partial_rounds=rounds,
+        mask_token_id=mask_id, device=dev)
+    assert got_ids == ref_ids and got_conf == ref_conf
+    assert sum(ref_conf) == min(draft_len, 1 + rounds)
+    assert eo.generate_partial_draft_rounds_for_selection(None, prompt, max_new_tokens=0, partial_rounds=3,
+                                                          mask_token_id=mask_id) == ([], [])
+
+
+def test_partial_draft_round_confirms_one_position(dev):
+    """One round on the device: exactly one masked position changes, the transfer mask names it, and a block
+    without masks is left alone."""
+    from prefilling_dllm_amd import engine_ops as eo
+    vocab, mask_id, n, d = 500, 500, 6, 8
+    model = _toy_model(vocab, 3)
+    block = torch.full((d,), mask_id, dtype=torch.int64, device=dev)
+    ids = torch.cat([torch.arange(n, device=dev), block])
+    tr = eo.partial_draft_round(model(ids).to(dev), block, prompt_len=n, mask_token_id=mask_id, first=True)
+    assert tr.cpu().tolist() == [True] + [False] * (d - 1) and int((block != mask_id).sum()) == 1
+    before = block.clone()
+    tr = eo.partial_draft_round(model(torch.cat([ids[:n], block])).to(dev), block, prompt_len=n, mask_token_id=mask_id)
+    assert int(tr.sum()) == 1 and int((block != before).sum()) == 1 and bool((block[tr] != mask_id).all())
+    full = torch.arange(d, dtype=torch.int64, device=dev)
+    tr = eo.partial_draft_round(model(torch.cat([ids[:n], full])).to(dev), full, prompt_len=n, mask_token_id=mask_id)
+    assert int(tr.sum()) == 0 and full.cpu().tolist() == list(range(d))
+    with pytest.raises(ValueError):
+        eo.partial_draft_round(model(ids).to(dev)[:-1], block, prompt_len=n, mask_token_id=mask_id)
+
+
 def test_rope_matches_reference_formula(dev):
     gen = torch.Generator().manual_seed(14)
     cs = ref_ops.rope_cos_sin_cache(128, 40000, base=1000000.0)

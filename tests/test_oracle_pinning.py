@@ -458,3 +458,46 @@ def test_prefill_sparse_reduces_to_known_cases():
     # a selection shorter than the sequence: anchors past its end are not valid (replace: no correction there)
     g_short = ref_ops.prefill_sparse_attention(q, k, v, causal, keep, rep, selection_outputs=dense[:8])
     assert (g_short[:8] - got[:8]).abs().max() < 1e-5 and (g_short[8:] - sub[8:]).abs().max() < 1e-6
+
+
+def test_partial_draft_rounds_hand_trace():
+    """fastdllm_engine.py:1013-1059 on a hand-computed trace.  Vocabulary of 5, prompt of 2, draft of 4, mask id 4.
+    The stand-in model returns fixed rows: the logits row at position p decides block position p - prompt_len + 1
+    (the shift).  Row sharpness: block position 0 <- row 1 (weak), 1 <- row 2 (sharpest), 2 <- row 3 and 3 <- row 4
+    (equal, medium).  Position 0 is confirmed first although it is the weakest; then position 1; then the tie of
+    positions 2 and 3 goes to position 2; a fourth round takes 3; a fifth finds no mask."""
+    import torch
+    rows = torch.zeros(6, 5)
+    rows[1, 3] = 0.5     # -> block position 0: token 3
+    rows[2, 1] = 9.0     # -> block position 1: token 1
+    rows[3, 2] = 4.0     # -> block position 2: token 2
+    rows[4, 0] = 4.0     # -> block position 3: token 0 (same confidence as position 2)
+    calls = []
+
+    def logits_of(ids):
+        calls.append(list(ids))
+        return rows.clone()
+
+    ids, conf = ref_ops.partial_draft_rounds(logits_of, [7, 8], 4, 0, 4)
+    assert ids == [3, 4, 4, 4] and conf == [True, False, False, False]
+    ids, conf = ref_ops.partial_draft_rounds(logits_of, [7, 8], 4, 1, 4)
+    assert ids == [3, 1, 4, 4] and conf == [True, True, False, False]
+    ids, conf = ref_ops.partial_draft_rounds(logits_of, [7, 8], 4, 2, 4)
+    assert ids == [3, 1, 2, 4] and conf == [True, True, True, False]
+    calls.clear()
+    ids, conf = ref_ops.partial_draft_rounds(logits_of, [7, 8], 4, 9, 4)
+    assert ids == [3, 1, 2, 0] and conf == [True] * 4
+    assert len(calls) == 4 and calls[-1] == [7, 8, 3, 1, 2, 4]     # stops when no mask is left
+    assert ref_ops.partial_draft_rounds(logits_of, [7, 8], 0, 3, 4) == ([], [])
+
+
+def test_assemble_global_keep_indices_hand_listed():
+    """fastdllm_engine.py:1524-1546: prompt of 12, chunks [2,5) and [5,9) (adjacent), 2 heads.  Head 0 keeps {2,4}
+    and {5,8}, head 1 keeps {3,4} and {6,7}; positions 0-1 and 9-11 lie outside every chunk."""
+    keeps = [[[[2, 4], [3, 4]], [[5, 8], [6, 7]]], []]
+    out = ref_ops.assemble_global_keep_indices(keeps, [(2, 5), (5, 9)], 12, 2)
+    assert out[0] == [[0, 1, 2, 4, 5, 8, 9, 10, 11], [0, 1, 3, 4, 6, 7, 9, 10, 11]]
+    assert out[1] == [list(range(12)), list(range(12))]
+    # a chunk that starts at 0 and one that ends at the prompt end: no gap, no tail
+    out = ref_ops.assemble_global_keep_indices([[[[0]], [[3]]]], [(0, 2), (2, 4)], 4, 1)
+    assert out == [[[0, 3]]]
