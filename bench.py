@@ -4,13 +4,16 @@
 Workload (BASELINE.json configs[2], "C3"): one denoise step = the attention of all 28 layers for 8
 requests, each with 128 query + 32 response rows (Dream-7B GQA 28/4, d=128, bf16) over its
 top-K = 8 of 32 chunks compacted to 512 tokens (16 non-contiguous 256-token pages per request out
-of a shared, seeded page pool) plus the active block itself.  The prefix KV stays fixed over the
-steps.  Inputs are synthetic (N(0,1)/sqrt(128)) and resident in HBM before the timed region.
+of a shared, seeded page pool) plus the active block itself, preceded -- as in the reference's decode forward
+(attention_v4.py:328-331) -- by the paged store of the active block's K/V rows into the request's block page.
+The prefix KV stays fixed over the steps.  Inputs are synthetic (N(0,1)/sqrt(128)) and resident in HBM before
+the timed region.
 
 Prints ONE JSON line: metric = microseconds per denoise step (lower is better), with the roofline
 of the dominant kernel (attn_fwd_kernel) and the CPU oracle timed on a bounded sample next to it.
 """
 import argparse
+import collections
 import json
 import math
 import os
@@ -23,10 +26,27 @@ if ROOT not in sys.path:
 
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
 PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
-# L2-miss bytes of one launch (attention + merge kernels) of this workload under the default plan, from two
-# rocprofv3 --pmc runs (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration on a 1 GiB copy):
-# profiles/attn_fwd_kernel_c3_decode_hbm_traffic.txt
-MEASURED_TRAFFIC_BYTES = {160: 272.9e6}   # rows per request -> bytes per launch
+# L2-miss bytes of one launch (attention + merge kernels) of this workload, from two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE, scaled by what the same counters read for a plain copy).  The summary of those runs
+# names the launch plan it was taken on ("plan: ..." as pdllm_attn_plan_describe prints it) and the resulting
+# figure ("traffic_bytes_per_launch: ..."); the figure is reported only while the library still picks that plan.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "attn_fwd_kernel_c3_decode_hbm_traffic.txt")
+
+
+def measured_traffic(plan_text):
+    """Bytes per launch from the committed counter summary, or None when it was taken on another plan."""
+    try:
+        lines = open(TRAFFIC_PROFILE).read().splitlines()
+    except OSError:
+        return None
+    plan = [ln.split(":", 1)[1].strip() for ln in lines if ln.startswith("plan:")]
+    val = [ln.split(":", 1)[1].strip() for ln in lines if ln.startswith("traffic_bytes_per_launch:")]
+    if len(plan) != 1 or len(val) != 1 or plan[0] != plan_text:
+        return None
+    return float(val[0])
+
+
+Layer = collections.namedtuple("Layer", "store attn")   # one layer of a step (store: a separate call, if any)
 
 HQ, HKV, D, PAGE = 28, 4, 128, 256
 LAYERS, N_REQ, N_CHUNKS, TOPK, CHUNK_TOKENS = 28, 8, 32, 8, 512
@@ -37,13 +57,13 @@ def build_workload(torch, dev, q_len=Q_LEN, layers=LAYERS, n_req=N_REQ, seed=0):
     g = torch.Generator(device="cpu").manual_seed(seed)
     pages_per_req = N_CHUNKS * CHUNK_TOKENS // PAGE            # logical pages of a request's prefix
     sel_pages = TOPK * CHUNK_TOKENS // PAGE                    # 16 pages actually read
-    n_pages = n_req * pages_per_req + 1
+    n_pages = n_req * pages_per_req + 1 + n_req                # + one block page per request for the active rows
     std = 1.0 / math.sqrt(D)
     gd = torch.Generator(device=dev).manual_seed(seed)
     kv = torch.empty((2, layers, n_pages, PAGE, HKV, D), dtype=torch.bfloat16, device=dev)
     for l in range(layers):  # fill per layer to bound the fp32 temporary
         kv[:, l] = (torch.randn((2, n_pages, PAGE, HKV, D), generator=gd, device=dev) * std).to(torch.bfloat16)
-    perm = torch.randperm(n_pages, generator=g)
+    perm = torch.randperm(n_pages - n_req, generator=g)
     block_table = torch.stack([perm[r * pages_per_req:(r + 1) * pages_per_req] for r in range(n_req)]).to(torch.int32)
     ptr, start, length = [0], [], []
     for r in range(n_req):
@@ -59,7 +79,10 @@ def build_workload(torch, dev, q_len=Q_LEN, layers=LAYERS, n_req=N_REQ, seed=0):
     vn = (torch.randn((layers, n_tok, HKV, D), generator=gd, device=dev) * std).to(torch.bfloat16)
     out = torch.empty_like(q)
     qsl = torch.arange(0, n_tok + 1, q_len, dtype=torch.int32, device=dev)
-    return dict(kv=kv, block_table=block_table.to(dev), ranges=(mk(ptr), mk(start), mk(length), TOPK), q=q, kn=kn,
+    # slot of active row i of request r: offset i of the request's block page (the pages behind the prefix pool)
+    block_page = torch.arange(n_pages - n_req, n_pages, dtype=torch.int32)
+    store_slots = (block_page.repeat_interleave(q_len) * PAGE + torch.arange(q_len, dtype=torch.int32).repeat(n_req))
+    return dict(store_slots=store_slots.to(dev), kv=kv, block_table=block_table.to(dev), ranges=(mk(ptr), mk(start), mk(length), TOPK), q=q, kn=kn,
                 vn=vn, out=out, qsl=qsl, q_len=q_len, ctx=TOPK * CHUNK_TOKENS, n_req=n_req, layers=layers,
                 ranges_host=[[(start[i], length[i]) for i in range(ptr[r], ptr[r + 1])] for r in range(n_req)],
                 sel_pages=sel_pages)
@@ -67,8 +90,9 @@ def build_workload(torch, dev, q_len=Q_LEN, layers=LAYERS, n_req=N_REQ, seed=0):
 
 def algorithmic_work(q_len, ctx, n_req):
     """Algorithmic work of one launch (= one layer, all requests): bytes = K/V pages of the selected keys + new K/V
-    + Q read + output written; FLOPs = 4 * rows * keys * d * heads (QK^T and PV, multiply and add)."""
-    by = n_req * (2 * ctx * HKV * D * 2 + 2 * q_len * HKV * D * 2 + 2 * q_len * HQ * D * 2)
+    read (once for the store and the attention) and written to the block page + Q read + output written;
+    FLOPs = 4 * rows * keys * d * heads (QK^T and PV, multiply and add)."""
+    by = n_req * (2 * ctx * HKV * D * 2 + 2 * 2 * q_len * HKV * D * 2 + 2 * q_len * HQ * D * 2)
     fl = n_req * 4 * q_len * (ctx + q_len) * D * HQ
     return by, fl
 
@@ -79,18 +103,21 @@ def prepare(ops, w, rows_per_group=0, num_splits=0, tiles_per_workgroup=0):
     table = ops.new_slot_table(w["n_req"], w["ctx"], w["q"].device)
     preps = []
     for l in range(w["layers"]):
-        preps.append(ops.PreparedAttention(w["q"][l], w["kn"][l], w["vn"][l], w["kv"][0, l], w["kv"][1, l],
+        preps.append(Layer(None, ops.PreparedAttention(w["q"][l], w["kn"][l], w["vn"][l], w["kv"][0, l], w["kv"][1, l],
                                            w["block_table"], w["qsl"], max_q_len=w["q_len"], max_ctx_len=w["ctx"],
                                            ranges=w["ranges"], out=w["out"][l], rows_per_group=rows_per_group,
                                            num_splits=num_splits, slot_table=table,
-                                           tiles_per_workgroup=tiles_per_workgroup))
+                                           tiles_per_workgroup=tiles_per_workgroup,
+                                           active_slot_mapping=w["store_slots"])))
     return preps
 
 
 def run_step(preps, stream):
-    preps[0].build_slot_table(stream)
+    """One denoise step: the slot table once, then per layer one library call = the store of the active K/V rows
+    and the attention."""
+    preps[0].attn.build_slot_table(stream)
     for p in preps:
-        p.run(stream)
+        p.attn.run(stream)
 
 
 def time_steps(torch, preps, steps, warmup):
@@ -298,6 +325,12 @@ def main():
     tflops = fl / launch_s / 1e12
     gbs = by / launch_s / 1e9
 
+    # the active rows of layer 0 now sit in the block pages
+    stored = w["kv"][0, 0].view(-1, HKV, D)[w["store_slots"].long()]
+    if not torch.equal(stored, w["kn"][0]):
+        print("bench.py: the active K rows were not stored into the block pages", file=sys.stderr)
+        sys.exit(4)
+
     # parity spot check of the timed outputs against the oracle (layer 0), and the CPU baseline
     cpu = None
     if not args.no_cpu:
@@ -316,6 +349,7 @@ def main():
 
     rows, splits = ops.attention_plan(w["n_req"], HQ, HKV, max_q_len=w["q_len"], max_ctx_len=w["ctx"],
                                       num_splits=args.num_splits, rows_per_group=args.rows_per_group)
+    plan_text = preps[0].attn.describe_plan()
     line = {
         "metric": "us/denoise-step sparse-KV attention, 32K prefix top-K=8 (28 layers, 8 requests, 160 rows)",
         "value": us_per_step, "unit": "us/step", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -326,8 +360,8 @@ def main():
                    "rows_per_workgroup": rows, "kv_splits": splits},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(w["q_len"]) if not (args.rows_per_group or args.num_splits or args.tiles_per_wg) else None,
-                     "kernel": "attn_fwd_kernel", "avg_launch_us": launch_s * 1e6,
+                     "traffic": measured_traffic(plan_text), "plan": plan_text,
+                     "kernel": plan_text.split()[0], "avg_launch_us": launch_s * 1e6,
                      "algorithmic_flops_per_launch": fl, "algorithmic_bytes_per_launch": by},
         "hbm": {"achieved_GBps": gbs, "peak_GBps": PEAK_HBM_GBS, "frac": gbs / PEAK_HBM_GBS},
         "cpu_baseline": cpu,

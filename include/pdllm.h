@@ -146,6 +146,13 @@ typedef struct pdllm_attn_desc {
    * and start the next; columns cut into pieces are merged from fp32 partials in the workspace.
    * Overrides num_splits. */
   int32_t tiles_per_workgroup;
+  /* optional, pdllm_sparse_decode_attn only: [n_tokens] cache slots (page * page_size + offset) of the active
+   * rows.  When not NULL the call also performs store_kvcache_unified_layout of k_new / v_new
+   * (attention_v4.py:328-331, OPS/kv_cache_kernels.py:150-172: slot < 0 or beyond the cache skips the row; fp8
+   * pages are quantised with the page scales) -- the store and the attention of the reference's decode forward in
+   * one call.  The cache must be the contiguous unified layout; the slots must not lie in the visible prefix of
+   * this call (they are the block's own pages, behind it). */
+  const int32_t* active_slot_mapping;
 } pdllm_attn_desc;
 
 /* Bytes of workspace pdllm_sparse_decode_attn needs for this descriptor: split-KV partials
@@ -185,6 +192,12 @@ int pdllm_attn_build_slot_table(const pdllm_attn_desc* desc, int32_t* table, int
  * rows per workgroup (32 * row blocks) and number of KV splits.  For tuning and tests. */
 int pdllm_attn_plan(const pdllm_attn_desc* desc, int32_t prefill, int32_t* rows_per_group,
                     int32_t* num_splits);
+
+/* The same plan as one line of text ("<kernel> kv=<dtype> row_blocks=J grid=.. span=.. head=.. set=.. tiles=..
+ * pieces=.."): which kernel runs and how the tiles of the launch are cut over workgroups.  No counterpart in the
+ * reference; it identifies a launch configuration so that measurements (profiles, counters) can be matched to the
+ * configuration they were taken on.  text receives at most text_bytes bytes including the terminating 0. */
+int pdllm_attn_plan_describe(const pdllm_attn_desc* desc, int32_t prefill, char* text, int32_t text_bytes);
 
 /* ------------------------------------------------------------------------- *
  * Chunk scoring and selection                                                *

@@ -47,6 +47,7 @@ class AttnDesc(C.Structure):
         ("page_size", i32), ("kv_dtype", i32), ("mask_mode", i32),
         ("num_splits", i32), ("rows_per_group", i32), ("sm_scale", f32),
         ("slot_table", vp), ("slot_table_stride", i64), ("tiles_per_workgroup", i32),
+        ("active_slot_mapping", vp),
     ]
 
 
@@ -62,6 +63,7 @@ SIGNATURES = {
     "pdllm_sparse_decode_attn": (C.c_int, [C.POINTER(AttnDesc), vp]),
     "pdllm_chunk_prefill_attn": (C.c_int, [C.POINTER(AttnDesc), vp, vp]),
     "pdllm_attn_plan": (C.c_int, [C.POINTER(AttnDesc), i32, C.POINTER(i32), C.POINTER(i32)]),
+    "pdllm_attn_plan_describe": (C.c_int, [C.POINTER(AttnDesc), i32, C.c_char_p, i32]),
     "pdllm_attn_slot_table_stride": (i64, [C.POINTER(AttnDesc)]),
     "pdllm_attn_build_slot_table": (C.c_int, [C.POINTER(AttnDesc), vp, i64, vp]),
     "pdllm_selfinfo_logprob": (C.c_int, [vp, i64, vp, i64, i64, vp, i64, vp, vp]),

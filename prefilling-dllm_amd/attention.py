@@ -48,7 +48,12 @@ class Attention(nn.Module):
         k_cache, v_cache = self.k_cache, self.v_cache
         has_cache = k_cache.numel() > 0 and v_cache.numel() > 0
 
-        if has_cache and context.need_kv_cache_store:
+        # A decode step over a cached prefix stores its active rows inside the attention call (their slots lie
+        # behind the context the same call reads, ENG:497); every other case stores first, as the reference does.
+        max_ctx = 0 if context.is_prefill else int(context.max_context_len) or max(int(context.max_seqlen_k) - 1, 0)
+        store_in_call = (has_cache and context.need_kv_cache_store and not context.is_prefill and max_ctx > 0
+                         and context.slot_mapping is not None)
+        if has_cache and context.need_kv_cache_store and not store_in_call:
             ops.store_kvcache_unified_layout(k, v, k_cache, v_cache, context.slot_mapping, self.model_type, context)
 
         mask_mode, dense = context.mask_kind, None
@@ -73,12 +78,12 @@ class Attention(nn.Module):
                 o = ops.chunk_prefill_attention(q, k, v, context.cu_seqlens_q, max_seqlen=int(context.max_seqlen_q),
                                                 causal=(mask_mode == "causal"), sm_scale=self.scale)
         else:
-            max_ctx = int(context.max_context_len) or max(int(context.max_seqlen_k) - 1, 0)
             o = ops.sparse_decode_attention(q, k, v, k_cache if has_cache else None, v_cache if has_cache else None,
                                             context.block_tables, context.cu_seqlens_q,
                                             max_q_len=int(context.max_seqlen_q), max_ctx_len=max_ctx if has_cache else 0,
                                             context_lens=context.context_lens, ranges=context.ranges,
-                                            mask_mode=mask_mode, mask=dense, sm_scale=self.scale)
+                                            mask_mode=mask_mode, mask=dense, sm_scale=self.scale,
+                                            active_slot_mapping=context.slot_mapping if store_in_call else None)
             o = self._maybe_apply_decode_delta(o, q, k, v, context, mask_mode, dense)
         return o.view(-1, self.num_heads * self.head_dim)
 

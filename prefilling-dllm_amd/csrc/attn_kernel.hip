@@ -26,7 +26,7 @@
 //   otherwise); the row addresses come from the slot table that attn_slot_table_kernel builds
 //   from the page table and the chunk ranges once per step, read two to three tiles ahead.
 //   Rows are 256 bytes = 16 chunks; chunk c of row r is stored at position
-//   c ^ rotl4(r & 15), which makes the 128-bit K operand reads and the transposing
+//   c ^ swz(r) (attn_common.h), which makes the 128-bit K operand reads and the transposing
 //   ds_read_b64_tr_b16 V operand reads bank-conflict free.
 //   S^T = K Q^T and O^T += V^T P^T use v_mfma_f32_32x32x16_bf16; in the S^T accumulator
 //   layout a lane holds 16 keys of one query, so softmax statistics are lane-local plus
@@ -41,6 +41,7 @@
 //   tiles from one source, in which the mask, end-of-piece and copy-source decisions are
 //   compile-time constants (a third fewer instructions per tile).
 
+#include <cstdio>
 #include <type_traits>
 
 #include "attn_common.h"
@@ -1067,12 +1068,36 @@ struct MergeParams {
   const int* q_start_loc;
   long o_stride, n_tokens;
   int n_req, max_q_len, Hq, Hkv, rows_per_group, row_tiles, t_lin, span, max_pieces, reversed, head;
+  // paged store of the active rows (bf16, unified layout) by the first store_blocks workgroups of the launch (they
+  // start first and their round trip to memory overlaps the merge); store_blocks == 0: no store
+  int store_blocks;
+  const int* store_slots;
+  const uint4* k_new;
+  const uint4* v_new;
+  uint4* k_cache;
+  uint4* v_cache;
+  long kn_stride16, vn_stride16, n_slots;  // strides in 16-byte units
 };
 
 __global__ __launch_bounds__(256) void attn_merge_kernel(const MergeParams m) {
+  if ((int)blockIdx.x < m.store_blocks) {
+    // store_kvcache of the active rows: one 16-byte chunk of a K row and of a V row per thread
+    const int cpr = m.Hkv * (kD / 8);  // chunks per token row
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    const long tok = idx / cpr;
+    const int ch = (int)(idx - tok * cpr);
+    if (tok >= m.n_tokens) return;
+    const long slot = m.store_slots[tok];
+    if (slot < 0 || slot >= m.n_slots) return;
+    const uint4 kv = m.k_new[tok * m.kn_stride16 + ch];
+    const uint4 vv = m.v_new[tok * m.vn_stride16 + ch];
+    m.k_cache[slot * cpr + ch] = kv;
+    m.v_cache[slot * cpr + ch] = vv;
+    return;
+  }
   // 32 lanes per row (4 columns each), 8 rows per workgroup
   const int l = threadIdx.x & 31;
-  const long row = (long)blockIdx.x * 8 + (threadIdx.x >> 5);
+  const long row = (long)((int)blockIdx.x - m.store_blocks) * 8 + (threadIdx.x >> 5);
   const long per_req = (long)m.max_q_len * m.Hq;
   if (row >= per_req * m.n_req) return;
   const int req = (int)(row / per_req);
@@ -1191,6 +1216,17 @@ static int validate_desc(const pdllm_attn_desc* d, bool prefill) {
     if (d->cache_page_stride != d->cache_token_stride * d->page_size) return PDLLM_ERR_STRIDE;
     const uintptr_t palign = d->kv_dtype == PDLLM_KV_FP8_E4M3 ? 8 : 16;
     if (((uintptr_t)d->k_cache | (uintptr_t)d->v_cache) % palign) return PDLLM_ERR_STRIDE;
+  }
+  if (!prefill && d->active_slot_mapping != nullptr) {
+    // the store writes whole token rows of a contiguous unified cache
+    if (!d->k_cache || !d->v_cache) return PDLLM_ERR_NULL;
+    if (d->kv_dtype != PDLLM_KV_BF16 && d->kv_dtype != PDLLM_KV_FP8_E4M3) return PDLLM_ERR_DTYPE;
+    if (d->kv_dtype == PDLLM_KV_FP8_E4M3 && (!d->k_scale || !d->v_scale)) return PDLLM_ERR_NULL;
+    if (ilog2_exact(d->page_size) < 0 || d->n_pages <= 0) return PDLLM_ERR_SHAPE;
+    if (d->cache_head_stride != kD || d->cache_token_stride != hk ||
+        d->cache_page_stride != hk * d->page_size)
+      return PDLLM_ERR_STRIDE;
+    if (((uintptr_t)d->k_cache | (uintptr_t)d->v_cache | (uintptr_t)d->active_slot_mapping) % 4) return PDLLM_ERR_STRIDE;
   }
   if (has_cache && d->slot_table != nullptr) {
     if (d->slot_table_stride < slot_table_stride_for(d) || ((uintptr_t)d->slot_table % 4)) return PDLLM_ERR_STRIDE;
@@ -1461,15 +1497,47 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
 #undef PDLLM_LAUNCH
   st = launch_status();
   if (st != PDLLM_OK) return st;
+  // Paged store of the active rows (the reference stores them in front of the attention, attention_v4.py:328-331;
+  // the slots lie behind the visible prefix, so the order within the call does not matter).  With a merge launch
+  // the copy rides in that launch -- a kernel of its own between two attention launches costs more than the
+  // copy -- otherwise, and for fp8 pages, it is the store kernel.
+  const bool store = !prefill && d->active_slot_mapping != nullptr;
+  const bool store_in_merge = store && plan.max_pieces > 1 && d->kv_dtype == PDLLM_KV_BF16;
+  if (store && !store_in_merge) {
+    const int64_t row = (int64_t)d->num_kv_heads * d->head_dim;
+    const int64_t n_slots = d->n_pages * (int64_t)d->page_size;
+    if (d->kv_dtype == PDLLM_KV_BF16)
+      st = kv_store_launch(d->k_new, d->v_new, const_cast<void*>(d->k_cache), const_cast<void*>(d->v_cache),
+                           d->active_slot_mapping, d->n_tokens, row, d->kn_stride, d->vn_stride, n_slots, stream);
+    else
+      st = pdllm_kv_store_fp8(d->k_new, d->v_new, const_cast<void*>(d->k_cache), const_cast<void*>(d->v_cache),
+                              d->k_scale, d->v_scale, d->active_slot_mapping, d->n_tokens, row, d->kn_stride,
+                              d->vn_stride, n_slots, d->page_size, d->head_dim, d->scale_page_stride,
+                              d->scale_head_stride, stream);
+    if (st != PDLLM_OK) return st;
+  }
   if (plan.max_pieces > 1) {
-    MergeParams m;
+    MergeParams m = {};
     m.ws_o = p.ws_o; m.ws_lse = p.ws_lse; m.out = p.out; m.q_start_loc = p.q_start_loc;
     m.o_stride = p.o_stride; m.n_tokens = p.n_tokens;
     m.n_req = p.n_req; m.max_q_len = p.max_q_len; m.Hq = p.Hq; m.Hkv = p.Hkv;
     m.rows_per_group = 32 * plan.J; m.row_tiles = plan.row_tiles; m.reversed = p.mask_mode == PDLLM_MASK_CAUSAL;
     m.t_lin = plan.t_lin; m.span = plan.span; m.max_pieces = plan.max_pieces; m.head = plan.head;
     const long mrows = (long)d->n_req * d->max_q_len * d->num_q_heads;
-    hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((mrows + 7) / 8)), dim3(256), 0, stream, m);
+    const int merge_blocks = (int)((mrows + 7) / 8);
+    if (store_in_merge) {
+      m.store_slots = d->active_slot_mapping;
+      m.k_new = static_cast<const uint4*>(d->k_new);
+      m.v_new = static_cast<const uint4*>(d->v_new);
+      m.k_cache = static_cast<uint4*>(const_cast<void*>(d->k_cache));
+      m.v_cache = static_cast<uint4*>(const_cast<void*>(d->v_cache));
+      m.kn_stride16 = d->kn_stride / 8;
+      m.vn_stride16 = d->vn_stride / 8;
+      m.n_slots = d->n_pages * (int64_t)d->page_size;
+      const long chunks = d->n_tokens * d->num_kv_heads * (kD / 8);
+      m.store_blocks = (int)((chunks + 255) / 256);
+    }
+    hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)(merge_blocks + m.store_blocks)), dim3(256), 0, stream, m);
     st = launch_status();
   }
   return st;
@@ -1528,6 +1596,19 @@ extern "C" int pdllm_chunk_prefill_attn(const pdllm_attn_desc* desc, const int32
     if (rc != PDLLM_OK) return rc;
   }
   return pdllm::launch_attn(desc, true, hs);
+}
+
+extern "C" int pdllm_attn_plan_describe(const pdllm_attn_desc* desc, int32_t prefill, char* text, int32_t text_bytes) {
+  const int st = pdllm::validate_desc(desc, prefill != 0);
+  if (st != PDLLM_OK) return st;
+  if (text == nullptr || text_bytes <= 0) return PDLLM_ERR_NULL;
+  const pdllm::AttnPlan plan = pdllm::make_plan(desc, prefill != 0);
+  const bool fp8 = !prefill && desc->k_cache != nullptr && desc->max_ctx_len > 0 && desc->kv_dtype == PDLLM_KV_FP8_E4M3;
+  const char* kernel = plan.J == 8 && !fp8 ? "attn_fwd2_kernel" : "attn_fwd_kernel";
+  const int n = snprintf(text, (size_t)text_bytes, "%s kv=%s row_blocks=%d grid=%d span=%d head=%d set=%d tiles=%d pieces=%d",
+                         kernel, fp8 ? "fp8" : "bf16", plan.J, plan.grid, plan.span, plan.head, plan.wg_set,
+                         plan.t_lin, plan.max_pieces);
+  return n > 0 && n < text_bytes ? PDLLM_OK : PDLLM_ERR_SHAPE;
 }
 
 extern "C" int pdllm_attn_plan(const pdllm_attn_desc* desc, int32_t prefill, int32_t* rows_per_group,

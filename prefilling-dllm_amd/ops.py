@@ -239,8 +239,12 @@ def sparse_decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.T
                             sm_scale: Optional[float] = None, k_scale: Optional[torch.Tensor] = None,
                             v_scale: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                             num_splits: int = 0, rows_per_group: int = 0,
-                            tiles_per_workgroup: int = 0) -> torch.Tensor:
+                            tiles_per_workgroup: int = 0,
+                            active_slot_mapping: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the active block over [selected prefix pages || active block].
+
+    active_slot_mapping: int32 [n_tokens] cache slots of the active rows; when given the call also stores
+    k_new / v_new there (store_kvcache_unified_layout of the decode forward, attention_v4.py:328-331).
 
     The visible prefix of request r is either `context_lens[r]` leading tokens of its page
     table (the reference's decode context, attention_v4.py:368-397) or an explicit list of
@@ -273,6 +277,7 @@ def sparse_decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.T
     desc = _fill_desc(q, k_new, v_new, out, k_cache, v_cache, block_table, q_start_loc, ranges, mask, mode,
                       max_q_len, max_ctx_len, sm_scale, k_scale, v_scale, num_splits, rows_per_group,
                       tiles_per_workgroup)
+    active_slot_mapping = _slot_mapping_arg(desc, active_slot_mapping, n_tokens)
     need = lib.pdllm_attn_workspace_bytes(C.byref(desc))
     if need < 0:
         check(int(need), "sparse_decode_attention")
@@ -283,6 +288,21 @@ def sparse_decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.T
     return out
 
 
+def _slot_mapping_arg(desc: AttnDesc, slots: Optional[torch.Tensor], n_tokens: int) -> Optional[torch.Tensor]:
+    """Bind the cache slots of the active rows to the descriptor (the store rides in the attention call).  Returns
+    the tensor the descriptor points at; the caller keeps it alive until the launch has been enqueued."""
+    if slots is None:
+        return None
+    _need_cuda(slots)
+    if slots.numel() != n_tokens:
+        raise ValueError(f"active_slot_mapping must name one slot per active row: {slots.numel()} vs {n_tokens}")
+    if not desc.k_cache:
+        raise ValueError("active_slot_mapping needs a KV cache to store into")
+    slots = slots.to(torch.int32).contiguous()
+    desc.active_slot_mapping = slots.data_ptr()
+    return slots
+
+
 class PreparedAttention:
     """A filled attention descriptor bound to its tensors, for loops that run the same shapes
     again and again (every denoise step reuses the page table, ranges and buffers): `run()` is one
@@ -291,7 +311,7 @@ class PreparedAttention:
     def __init__(self, q, k_new, v_new, k_cache, v_cache, block_table, q_start_loc, *, max_q_len, max_ctx_len,
                  context_lens=None, ranges=None, mask_mode="full", mask=None, sm_scale=None, k_scale=None,
                  v_scale=None, out=None, num_splits=0, rows_per_group=0, workspace=None, slot_table=None,
-                 tiles_per_workgroup=0):
+                 tiles_per_workgroup=0, active_slot_mapping=None):
         """slot_table: an int32 tensor from `new_slot_table` shared by every layer of a step; the caller
         refreshes it with `build_slot_table()` of any one of the prepared layers whenever the page table
         or the ranges change.  Without it every `run()` rebuilds the table in its workspace."""
@@ -319,6 +339,7 @@ class PreparedAttention:
                                mask, mode, max_q_len, max_ctx_len,
                                1.0 / math.sqrt(d) if sm_scale is None else sm_scale, k_scale, v_scale,
                                num_splits, rows_per_group, tiles_per_workgroup)
+        active_slot_mapping = _slot_mapping_arg(self.desc, active_slot_mapping, n_tokens)
         self.slot_table = slot_table
         if slot_table is not None and k_cache is not None and max_ctx_len > 0:
             if slot_table.dtype != torch.int32 or slot_table.dim() != 2 or slot_table.stride(1) != 1:
@@ -334,7 +355,7 @@ class PreparedAttention:
             self.desc.workspace, self.desc.workspace_bytes = workspace.data_ptr(), int(need)
         # keep every tensor the descriptor points at alive
         self._keep = (q, k_new, v_new, k_cache, v_cache, block_table, q_start_loc, ranges, mask, k_scale, v_scale,
-                      workspace, slot_table)
+                      workspace, slot_table, active_slot_mapping)
         self._ref = C.byref(self.desc)
         self._fn = lib.pdllm_sparse_decode_attn
 
@@ -343,6 +364,12 @@ class PreparedAttention:
         if st != 0:
             check(st, "PreparedAttention.run")
         return self.out
+
+    def describe_plan(self) -> str:
+        """One line naming the kernel and the cut of the launch this descriptor leads to (pdllm_attn_plan_describe)."""
+        buf = C.create_string_buffer(256)
+        check(lib.pdllm_attn_plan_describe(self._ref, 0, buf, 256), "PreparedAttention.describe_plan")
+        return buf.value.decode()
 
     def build_slot_table(self, stream: Optional[int] = None) -> None:
         """(Re)build the shared slot table from this layer's page table and ranges."""

@@ -613,3 +613,44 @@ def test_seeded_random_ragged_requests_cut_ranges_and_dense_masks(dev):
         out = run_case(case, dev, mask_mode=mode, mask=mask, **plan)
         ref = oracle_case(case, mask_mode=mode, mask=mask)
         check(out, ref, what=f"case {i} lens {lens} plan {plan} mask {mode}")
+
+
+@pytest.mark.parametrize("fp8", [False, True], ids=["bf16", "fp8"])
+@pytest.mark.parametrize("plan", [dict(), dict(num_splits=1), dict(rows_per_group=256), dict(rows_per_group=32, num_splits=3)],
+                         ids=["default", "unsplit", "wide", "split3"])
+def test_active_rows_stored_inside_the_attention_call(dev, fp8, plan):
+    """desc.active_slot_mapping: the call stores k_new / v_new like store_kvcache_unified_layout
+    (attention_v4.py:328-331, OPS/kv_cache_kernels.py:150-172) and attends like the call without it.  The store is
+    compared bit for bit with the separate store operator on a copy of the cache; rows with slot -1 are skipped and
+    every other cache row stays as it was (with and without a merge launch, bf16 and fp8 pages)."""
+    ops = _ops()
+    case = configs.chunked_prefix_case(21, n_req=2, n_chunks=6, chunk_tokens=512, topk=3, q_len=40,
+                                       shared_prefix=False, fp8=fp8, extra_pages=3)
+    d = lambda t: None if t is None else t.to(dev)
+    n_tok = case.q.shape[0]
+    n_pages = case.k_cache.shape[0]
+    used = set(case.block_table.flatten().tolist())
+    free = [p for p in range(n_pages) if p not in used]
+    assert len(free) >= 2
+    slots = torch.cat([torch.arange(40, dtype=torch.int32) + free[r] * 256 + 7 for r in range(2)])
+    slots[3] = -1
+    slots[55] = -1
+    rp, rs, rl, mr = case.range_tensors()
+    kc, vc = d(case.k_cache), d(case.v_cache)
+    kc2, vc2 = kc.clone(), vc.clone()
+    args = (d(case.q), d(case.k_new), d(case.v_new))
+    kw = dict(max_q_len=case.max_q, max_ctx_len=case.max_ctx, ranges=(d(rp), d(rs), d(rl), mr),
+              k_scale=d(case.k_scale), v_scale=d(case.v_scale), **plan)
+    plain = ops.sparse_decode_attention(*args, kc2, vc2, d(case.block_table), d(case.q_start_loc), **kw)
+    ops.store_kvcache_unified_layout(args[1], args[2], kc2, vc2, d(slots), k_scale=d(case.k_scale), v_scale=d(case.v_scale))
+    fused = ops.sparse_decode_attention(*args, kc, vc, d(case.block_table), d(case.q_start_loc),
+                                        active_slot_mapping=d(slots), **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(fused, plain)
+    as_bits = lambda t: t.view(torch.uint8) if t.dtype != torch.bfloat16 else t.view(torch.int16)
+    assert torch.equal(as_bits(kc), as_bits(kc2)) and torch.equal(as_bits(vc), as_bits(vc2))
+    assert not torch.equal(as_bits(kc), as_bits(d(case.k_cache)))          # something was stored
+    check(fused.float().cpu(), oracle_case(case))
+    with pytest.raises(ValueError):
+        ops.sparse_decode_attention(*args, kc, vc, d(case.block_table), d(case.q_start_loc),
+                                    active_slot_mapping=d(slots[:-1]), **kw)
