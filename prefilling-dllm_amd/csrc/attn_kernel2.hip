@@ -149,8 +149,27 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
     const int kvh = (col / p.row_tiles) % p.Hkv;
     const int req = col / (p.row_tiles * p.Hkv);
 
+    // Everything the piece needs from memory before its first copy is requested here at once: the row range of
+    // the request, the number of prefix keys, and -- before that number is known -- the slot-table entries its
+    // first three tiles would use if they are prefix tiles (in-bounds reads of the request's table row, taken or
+    // dropped once the count has arrived).  One round trip to memory instead of three in a row.
     const int q0 = p.q_start_loc[req];
-    const int Sq = p.q_start_loc[req + 1] - q0;
+    const int q1 = p.q_start_loc[req + 1];
+    const int* tbl = p.slot_table != nullptr ? p.slot_table + (long)req * p.slot_stride : nullptr;
+    int ctx_total = tbl != nullptr ? tbl[p.slot_stride - 1] : 0;
+    const int lane_row = 4 * wave + (lane >> 4);  // row (of every group of 4 NW rows) this lane copies
+    int spec[3][16 / NW];
+    if (tbl != nullptr) {
+      const int last = (int)p.slot_stride - 2;
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+#pragma unroll
+        for (int i = 0; i < 16 / NW; ++i) {
+          const int idx = (tb + j) * kKT + 4 * NW * i + lane_row;
+          spec[j][i] = tbl[idx < last ? idx : last];
+        }
+    }
+    const int Sq = q1 - q0;
     if (q0 < 0 || Sq <= 0 || (long)q0 + Sq > p.n_tokens || Sq > p.max_q_len) continue;
     const int rows = Sq * G;
     const int row0 = row_tile * 32 * J;
@@ -160,8 +179,6 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
     const int l32e = lane_e & 31;
     const int he = lane_e >> 5;
 
-    const int* tbl = p.slot_table != nullptr ? p.slot_table + (long)req * p.slot_stride : nullptr;
-    int ctx_total = tbl != nullptr ? tbl[p.slot_stride - 1] : 0;
     ctx_total = __builtin_amdgcn_readfirstlane(ctx_total);
     const int Tc = (ctx_total + kKT - 1) / kKT;
     int Sa = Sq;
@@ -230,7 +247,6 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
     };
 
     // ---- K/V copies HBM -> LDS: this wave moves rows 4*NW*i + 4*wave + lane/16 of a tile, i < kDmaGroups ----
-    const int lane_row = 4 * wave + (lane >> 4);
     const int lane_ch = (lane & 15) ^ swz(lane_row);
     const unsigned cache_row16 = (unsigned)((p.cache_token_stride * 2) >> 4);  // 16-byte units
     const unsigned kn_row16 = (unsigned)((p.kn_stride * 2) >> 4);
@@ -238,10 +254,11 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
     int nslot[kDmaGroups];  // slots of the next K tile to copy
     int nsv[kDmaGroups];    // slots of the next V tile to copy
     int nnext[kDmaGroups];  // slots of the tile after those, on their way from the slot table
-    auto load_slots = [&](int (&dst)[kDmaGroups], int t) __attribute__((always_inline)) {
+    // j >= 0: tile t is the piece's j-th tile, whose table entries have been requested above
+    auto load_slots = [&](int (&dst)[kDmaGroups], int t, int j = -1) __attribute__((always_inline)) {
       if (t < Tc) {
 #pragma unroll
-        for (int i = 0; i < kDmaGroups; ++i) dst[i] = tbl[t * kKT + 4 * NW * i + lane_row];
+        for (int i = 0; i < kDmaGroups; ++i) dst[i] = j >= 0 ? spec[j][i] : tbl[t * kKT + 4 * NW * i + lane_row];
       } else {
         // padding rows copy the first row of the tile, tiles past the end of the column the last tile's rows: always
         // a valid row (they are masked, or never read)
@@ -332,8 +349,14 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
         for (int w = 0; w < 8; ++w) Pw[1][rb][w] = 0u;  // "the block before the first one": contributes nothing
       bool pending = false;   // the accumulators still have to be rescaled by alpha[]
       float alpha[NB];
+      float negM[NB];   // -M, or 0 while M is still -inf (then every score is -inf as well)
+      float Mneed[NB];  // M + slack: a block maximum above it moves the running maximum
 #pragma unroll
-      for (int rb = 0; rb < NB; ++rb) alpha[rb] = 1.f;
+      for (int rb = 0; rb < NB; ++rb) {
+        alpha[rb] = 1.f;
+        negM[rb] = 0.f;
+        Mneed[rb] = -INFINITY;
+      }
 
       // One step of the pipeline.  E = parity of block k inside its tile (0: first 32 keys).
       //   softmax of block k: scores S[E] -> Pw[E]          (masks: lim[rb] = visible keys of the tile, mrow)
@@ -387,7 +410,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
 #pragma unroll
           for (int i = 2; i < 16; i += 2) m0 = fmaxf(fmaxf(m0, Sc[rb][i]), Sc[rb][i + 1]);
           mx[rb] = half_swap_max(m0) * c;  // log2 units; -inf (nothing visible) stays -inf
-          need = need || mx[rb] > M[rb] + kRescaleSlack;
+          need = need || mx[rb] > Mneed[rb];
         }
         if (__builtin_amdgcn_ballot_w64(need) != 0) {
 #pragma unroll
@@ -397,12 +420,11 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
             alpha[rb] = a;
             M[rb] = Mn;
             l[rb] *= a;
+            negM[rb] = (Mn == -INFINITY) ? 0.f : -Mn;
+            Mneed[rb] = Mn + kRescaleSlack;
           }
           pending = true;
         }
-        float negM[NB];
-#pragma unroll
-        for (int rb = 0; rb < NB; ++rb) negM[rb] = (M[rb] == -INFINITY) ? 0.f : -M[rb];
         const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
         float psum[NB];
 #pragma unroll
@@ -422,7 +444,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
         // scores 2 (s % 8) and + 1).  The scores and the intermediate results pass through (empty) asm statements
         // of their half: that keeps the arithmetic there -- the instruction selector would otherwise gather all of
         // it in one place.
-        float xprev = 0.f;  // NB == 1: the first probability of a pair, kept for one slot
+        float xa = 0.f, xb = 0.f;  // the probabilities of the pair that is packed next
 #pragma unroll
         for (int s = 0; s < 16; ++s) {
           const int f = s >> 1;
@@ -451,17 +473,24 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
             const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
             frag = __builtin_bit_cast(bf16x8, both);
           }
+          // The two probabilities of a pair are packed (and added to the row sum) one half-slot after the second
+          // exponential: a result of the transcendental unit read by the very next instruction costs a wait state.
           if constexpr (NB == 2) {
             const int prb = s >> 3, pi = 2 * (s & 7);
             float e0 = Sc[prb][pi], e1 = Sc[prb][pi + 1];
-            // ---- first half: MFMA of row block 0, first probability ----
-            asm volatile("" : "+v"(e0), "+v"(psum[prb]));
+            // ---- first half: MFMA of row block 0, pack of the previous pair, first probability ----
+            asm volatile("" : "+v"(e0), "+v"(psum[0]), "+v"(psum[1]), "+v"(xa), "+v"(xb));
             if ((s & 1) == 0) Sn[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, Q[0][f], Sn[0], 0, 0, 0);
             else O[0][f & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, p_frag(E ^ 1, 0, f >> 2), O[0][f & 3], 0, 0, 0);
-            float x0 = exp2s(e0, prb);
+            if (s > 0) {
+              const bf16x2 pv2 = {(__bf16)xa, (__bf16)xb};
+              psum[(s - 1) >> 3] = __builtin_amdgcn_fdot2_f32_bf16(pv2, ones, psum[(s - 1) >> 3], false);
+              Pw[E][(s - 1) >> 3][(s - 1) & 7] = __builtin_bit_cast(uint32_t, pv2);
+            }
+            xa = exp2s(e0, prb);
             __builtin_amdgcn_sched_barrier(0);
-            // ---- second half: MFMA of row block 1, second probability, pack, row sum; next fragment ----
-            asm volatile("" : "+v"(e1), "+v"(x0));
+            // ---- second half: MFMA of row block 1, second probability; next fragment ----
+            asm volatile("" : "+v"(e1), "+v"(xa));
             if ((s & 1) == 0) {
               Sn[NB - 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, Q[NB - 1][f], Sn[NB - 1], 0, 0, 0);
               if (f + 2 < 8) rdk(kf[(f + 2) % 3], E ^ 1, f + 2);
@@ -471,29 +500,36 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
                   __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, p_frag(E ^ 1, NB - 1, f >> 2), O[NB - 1][f & 3], 0, 0, 0);
               if (f + 2 < 8) { rdv(vlo[f & 1], E ^ 1, f + 2, 0); rdv(vhi[f & 1], E ^ 1, f + 2, 1); }
             }
-            const float x1 = exp2s(e1, prb);
-            const bf16x2 pv2 = {(__bf16)x0, (__bf16)x1};
-            psum[prb] = __builtin_amdgcn_fdot2_f32_bf16(pv2, ones, psum[prb], false);
-            Pw[E][prb][s & 7] = __builtin_bit_cast(uint32_t, pv2);
+            xb = exp2s(e1, prb);
           } else {
-            // one row block per wave: one MFMA and one probability per slot, a pair is packed in every odd slot
+            // one row block per wave: one MFMA and one probability per slot; the pair of slots s - 2, s - 1 is
+            // packed in the even slot s
             float e = Sc[0][s];
-            asm volatile("" : "+v"(e), "+v"(psum[0]), "+v"(xprev));
+            asm volatile("" : "+v"(e), "+v"(psum[0]), "+v"(xa), "+v"(xb));
             if ((s & 1) == 0) {
               Sn[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, Q[0][f], Sn[0], 0, 0, 0);
+              if (s > 0) {
+                const bf16x2 pv2 = {(__bf16)xa, (__bf16)xb};
+                psum[0] = __builtin_amdgcn_fdot2_f32_bf16(pv2, ones, psum[0], false);
+                Pw[E][0][(s >> 1) - 1] = __builtin_bit_cast(uint32_t, pv2);
+              }
               if (f + 2 < 8) rdk(kf[(f + 2) % 3], E ^ 1, f + 2);
               dma(f);
-              xprev = exp2s(e, 0);
+              xa = exp2s(e, 0);
             } else {
               O[0][f & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, p_frag(E ^ 1, 0, f >> 2), O[0][f & 3], 0, 0, 0);
               if (f + 2 < 8) { rdv(vlo[f & 1], E ^ 1, f + 2, 0); rdv(vhi[f & 1], E ^ 1, f + 2, 1); }
-              const float x1 = exp2s(e, 0);
-              const bf16x2 pv2 = {(__bf16)xprev, (__bf16)x1};
-              psum[0] = __builtin_amdgcn_fdot2_f32_bf16(pv2, ones, psum[0], false);
-              Pw[E][0][s >> 1] = __builtin_bit_cast(uint32_t, pv2);
+              xb = exp2s(e, 0);
             }
           }
           __builtin_amdgcn_sched_barrier(0);
+        }
+        {
+          // the last pair
+          asm volatile("" : "+v"(xa), "+v"(xb));
+          const bf16x2 pv2 = {(__bf16)xa, (__bf16)xb};
+          psum[NB - 1] = __builtin_amdgcn_fdot2_f32_bf16(pv2, ones, psum[NB - 1], false);
+          Pw[E][NB - 1][7] = __builtin_bit_cast(uint32_t, pv2);
         }
 #pragma unroll
         for (int rb = 0; rb < NB; ++rb) {
@@ -515,7 +551,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
       };
 
       // ---- prologue: K(T0), V(T0), K(T0+1); scores of the first block ----
-      load_slots(nslot, T0);
+      load_slots(nslot, T0, 0);  // (T0 == tb: the piece has tiles)
 #pragma unroll
       for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
       {
@@ -528,14 +564,14 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
       {
         // (like the copies inside the loop, issued whether or not the piece has a second tile: the slots loaded for a
         // tile and the source chosen for it always belong together)
-        load_slots(nslot, T0 + 1);
+        load_slots(nslot, T0 + 1, 1);
         const TileSrc sk = src_of(T0 + 1, kc_base, kn_base, kn_row16);
 #pragma unroll
         for (int i = 0; i < kDmaGroups; ++i) issue_k1(sk, 1, i);
       }
 #pragma unroll
       for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];  // slots of tile T0 + 1 for its V copy
-      load_slots(nslot, T0 + 2);
+      load_slots(nslot, T0 + 2, 2);
       build_mask(T0, 0);
       __builtin_amdgcn_s_waitcnt(0x0F70);
       __syncthreads();
