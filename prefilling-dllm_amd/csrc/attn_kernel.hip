@@ -1257,6 +1257,20 @@ static int dyn_lds_bytes(int J, int mask_mode) {
 // workgroup alone on a CU spends (fixed + blocks per wave) per tile; two workgroups sharing a CU
 // (at most 4 row blocks, LDS footprint <= 80 KB) overlap matrix and vector work and take kPair of the
 // serial time.  The most loaded CU sets the makespan.
+// Compute units of the current device (the planner balances over them); 256, an MI355X, when no device can be
+// asked -- sizes and plans can be queried on a machine without a GPU.
+static int compute_units() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   const int G = d->num_q_heads / d->num_kv_heads;
   const long rows = (long)d->max_q_len * G;
@@ -1265,7 +1279,7 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   const long T = (ctx + kKT - 1) / kKT + (d->max_q_len + kKT - 1) / kKT;
   const long units = (long)d->n_req * d->num_kv_heads;
   const bool fp8 = !prefill && d->k_cache != nullptr && d->max_ctx_len > 0 && d->kv_dtype == PDLLM_KV_FP8_E4M3;
-  const int cus = 256;
+  const int cus = compute_units();
   constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 1.5, kWide = 1.25;
   constexpr int kStaticLds = 66 * 1024;
   static const int js[] = {1, 2, 4, 5, 6, 8};
