@@ -1289,8 +1289,10 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   for (int ji = 0; ji < 6; ++ji) {
     const int J = js[ji];
     if (d->rows_per_group && d->rows_per_group != 32 * J) continue;
-    // 5 and 6 row blocks need more than 256 registers (one workgroup per CU): only on request
-    if (!d->rows_per_group && (J == 5 || J == 6)) continue;
+    // 5 and 6 row blocks need more than 256 registers (one workgroup per CU): on request, and for an fp8
+    // cache (which has no 8-block kernel) when they hold all rows of a (request, KV head) in one column
+    // where 4 blocks would leave a second, mostly empty one (160 rows of an MHA layer: 322 us against 362)
+    if (!d->rows_per_group && (J == 5 || J == 6) && !(fp8 && nblk > 4 && nblk <= J)) continue;
     if (J == 8 && fp8) continue;  // the 8-wave workgroup has no room for the fp8 staging registers
     if (J == 8 && prefill && !d->rows_per_group) continue;  // coarser causal staircase: measured slower
     const long row_tiles = (nblk + J - 1) / J;
