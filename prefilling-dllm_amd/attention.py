@@ -115,6 +115,24 @@ class Attention(nn.Module):
         state["max_abs"] = max(float(state.get("max_abs", 0.0)), delta_abs_max)
         state["anchor_count"] = int(state.get("anchor_count", 0)) + n_anchors
 
+    def _paged_prompt(self, state, full_k, full_v, extra: int):
+        """The layer's full prompt K/V [S, Hkv, d] as pages of a cache of its own (where the reference concatenates,
+        attention_v4.py:120-125) with room for `extra` more tokens.  The copy is kept in the state between steps and
+        made again when the prompt tensors change."""
+        page, n_prompt = 256, int(full_k.shape[0])
+        pages = (n_prompt + extra + page - 1) // page
+        key = (full_k.data_ptr(), full_v.data_ptr(), n_prompt, full_k._version, full_v._version)
+        held = state.setdefault("_paged_prompt", {})
+        ent = held.get(self.layer_idx)
+        if ent is None or ent[0] != key or ent[1].shape[0] < pages:
+            kc = torch.empty((pages, page, self.num_kv_heads, self.head_dim), dtype=full_k.dtype, device=full_k.device)
+            vc = torch.empty_like(kc)
+            kc.view(-1, self.num_kv_heads, self.head_dim)[:n_prompt].copy_(full_k)
+            vc.view(-1, self.num_kv_heads, self.head_dim)[:n_prompt].copy_(full_v)
+            ent = (key, kc, vc)
+            held[self.layer_idx] = ent
+        return ent[1], ent[2]
+
     def _maybe_apply_decode_delta(self, o, q, k_new, v_new, context, mask_mode="full", active_mask=None):
         """attention_v4.py:86-166.  The packed active rows are one sequence, as in the reference; active_mask is the
         [Nq, Nq] mask over the active keys (attention_v4.py:131-133 takes those columns of the block mask)."""
@@ -132,23 +150,38 @@ class Attention(nn.Module):
         if ap is None:
             return o
         stride, offset, left, right, direction = ap
-        # the full prompt K/V [S, Hkv, d] as pages of a cache of its own (one copy, where the reference concatenates)
-        n_prompt, page = int(full_k.shape[0]), 256
-        pages = (n_prompt + page - 1) // page
-        kc = torch.empty((pages, page, self.num_kv_heads, self.head_dim), dtype=k_new.dtype, device=k_new.device)
-        vc = torch.empty_like(kc)
-        kc.view(-1, self.num_kv_heads, self.head_dim)[:n_prompt].copy_(full_k)
-        vc.view(-1, self.num_kv_heads, self.head_dim)[:n_prompt].copy_(full_v)
         dev = q.device
+        n_prompt = int(full_k.shape[0])
+        anchors = torch.arange(offset, seq_len, stride, device=dev)
+        n_a = int(anchors.numel())
+        if mask_mode == "full" and active_mask is None and 0 < n_a < seq_len:
+            # Only the anchor rows are attended, as in the reference (attention_v4.py:127): the active K/V rows are
+            # appended to the paged copy of the prompt, so that every key is a prefix key and the anchors are a
+            # compact batch of queries whose own "active" keys are all masked.
+            kc, vc = self._paged_prompt(state, full_k, full_v, seq_len)
+            kc.view(-1, self.num_kv_heads, self.head_dim)[n_prompt:n_prompt + seq_len].copy_(k_new)
+            vc.view(-1, self.num_kv_heads, self.head_dim)[n_prompt:n_prompt + seq_len].copy_(v_new)
+            n_keys = n_prompt + seq_len
+            dense_a = ops.sparse_decode_attention(
+                q.index_select(0, anchors), k_new.index_select(0, anchors), v_new.index_select(0, anchors), kc, vc,
+                torch.arange(kc.shape[0], dtype=torch.int32, device=dev).view(1, -1),
+                torch.tensor([0, n_a], dtype=torch.int32, device=dev), max_q_len=n_a, max_ctx_len=n_keys,
+                context_lens=torch.tensor([n_keys], dtype=torch.int32, device=dev), mask_mode="dense",
+                mask=torch.zeros((n_a, n_a), dtype=torch.bool, device=dev), sm_scale=self.scale)
+            dense = torch.empty_like(o)   # only the anchor rows are read below
+            dense.index_copy_(0, anchors, dense_a)
+        else:
+            # a mask over the active keys applies to keys, not to rows: every active row goes through the kernel
+            kc, vc = self._paged_prompt(state, full_k, full_v, 0)
+            dense = ops.sparse_decode_attention(q, k_new, v_new, kc, vc,
+                                                torch.arange(kc.shape[0], dtype=torch.int32, device=dev).view(1, -1),
+                                                torch.tensor([0, seq_len], dtype=torch.int32, device=dev),
+                                                max_q_len=seq_len, max_ctx_len=n_prompt,
+                                                context_lens=torch.tensor([n_prompt], dtype=torch.int32, device=dev),
+                                                mask_mode=mask_mode, mask=active_mask, sm_scale=self.scale)
         one_seq = torch.tensor([0, seq_len], dtype=torch.int32, device=dev)
-        dense = ops.sparse_decode_attention(q, k_new, v_new, kc, vc,
-                                            torch.arange(pages, dtype=torch.int32, device=dev).view(1, -1), one_seq,
-                                            max_q_len=seq_len, max_ctx_len=n_prompt,
-                                            context_lens=torch.tensor([n_prompt], dtype=torch.int32, device=dev),
-                                            mask_mode=mask_mode, mask=active_mask, sm_scale=self.scale)
         scale = float(state.get("scale", 1.0))
         if state.get("debug", False):
-            anchors = torch.arange(offset, seq_len, stride, device=dev)
             delta = (dense.index_select(0, anchors) - o.index_select(0, anchors)) * scale
             self._debug_stats(state, float(delta.abs().max().item()) if delta.numel() else 0.0, int(anchors.numel()))
         return ops.anchor_delta_add(o, dense, one_seq, max_q_len=seq_len, stride=stride, anchor_offset=offset,

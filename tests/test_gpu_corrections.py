@@ -127,6 +127,22 @@ def test_decode_delta_layer(dev, state):
     assert (got - ref).abs().max() <= 3e-2, (got - ref).abs().max()
     if state.get("debug"):
         assert st["calls"] == 1 and st["nonzero_calls"] == 1 and st["anchor_count"] == len(ref_ops.anchor_windows(block, state)[0])
+    # the paged copy of the prompt is kept between steps and made again when the prompt changes in place
+    def again():
+        set_context_diffusion_lm(False, cu_seqlens_q=cu.to(dev), max_seqlen_q=block, max_seqlen_k=n_ctx + block,
+                                 block_tables=bt.to(dev), need_kv_cache_store=False, decode_delta_state=st,
+                                 ranges=(rp.to(dev), rs.to(dev), rl.to(dev), len(ranges[0])), max_context_len=n_ctx)
+        try:
+            return layer(q.to(dev).view(block, -1), k.to(dev).view(block, -1), v.to(dev).view(block, -1)) \
+                .view(block, Hq, d).float().cpu()
+        finally:
+            reset_context_diffusion_lm()
+    held = st["_paged_prompt"][1][1]
+    assert torch.equal(again(), got) and st["_paged_prompt"][1][1] is held
+    st["full_v"][1].mul_(-1.0)
+    ref_neg = ref_ops.decode_delta(base, q.float(), k.float(), v.float(), fk.float(), -fv.float(), state)
+    assert (again() - ref_neg).abs().max() <= 3e-2 and st["_paged_prompt"][1][1] is not held
+    st["full_v"][1].mul_(-1.0)
     # disabled or without a prompt for this layer: the plain decode result
     for off in (dict(st, enabled=False), dict(st, full_k=[None, None])):
         set_context_diffusion_lm(False, cu_seqlens_q=cu.to(dev), max_seqlen_q=block, max_seqlen_k=n_ctx + block,
