@@ -227,6 +227,17 @@ def test_fp8_pages_with_per_page_scale(dev):
     check(run_case(case, dev), oracle_case(case))
 
 
+@pytest.mark.parametrize("q_len,Hq,Hkv,blocks", [(160, 32, 32, 5), (176, 8, 8, 6), (90, 8, 4, 6), (65, 8, 4, 5)])
+def test_fp8_groups_of_five_and_six_row_blocks(dev, q_len, Hq, Hkv, blocks):
+    """fp8 pages have no 8-block kernel: 129-192 rows per (request, KV head) can run as one group of 5 or 6 row
+    blocks (the planner's choice for large shapes; forced here), MHA and grouped heads, cut and uncut."""
+    case = configs.chunked_prefix_case(21 + q_len, n_req=2, n_chunks=5, chunk_tokens=300, topk=3, q_len=q_len,
+                                       Hq=Hq, Hkv=Hkv, fp8=True)
+    ref = oracle_case(case)
+    for splits in (0, 1, 3):
+        check(run_case(case, dev, rows_per_group=32 * blocks, num_splits=splits), ref, what=f"splits={splits}")
+
+
 def test_fp8_codes_decode_like_torch(dev):
     """All 256 e4m3 codes through the kernel's dequantisation == torch.float8_e4m3fn -> float."""
     ops = _ops()

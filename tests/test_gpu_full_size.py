@@ -97,10 +97,14 @@ def test_config5_full_fp8_decode_layer_and_unmask(dev):
                                        Hkv=32, fp8=True, shared_prefix=True)
     d = lambda t: None if t is None else t.to(dev)
     rp, rs, rl, mr = case.range_tensors()
-    out = ops.sparse_decode_attention(d(case.q), d(case.k_new), d(case.v_new), d(case.k_cache), d(case.v_cache),
-                                      d(case.block_table), d(case.q_start_loc), max_q_len=case.max_q,
-                                      max_ctx_len=case.max_ctx, ranges=(d(rp), d(rs), d(rl), mr),
-                                      k_scale=d(case.k_scale), v_scale=d(case.v_scale)).float().cpu()
+    prep = ops.PreparedAttention(d(case.q), d(case.k_new), d(case.v_new), d(case.k_cache), d(case.v_cache),
+                                 d(case.block_table), d(case.q_start_loc), max_q_len=case.max_q,
+                                 max_ctx_len=case.max_ctx, ranges=(d(rp), d(rs), d(rl), mr),
+                                 k_scale=d(case.k_scale), v_scale=d(case.v_scale))
+    # 160 rows per (request, head) are five row blocks: one workgroup column each (four blocks would open a second,
+    # mostly empty group that reads the pages again)
+    assert "kv=fp8 row_blocks=5 " in prep.describe_plan(), prep.describe_plan()
+    out = prep.run().float().cpu()
     assert torch.isfinite(out).all()
     # oracle on the first and last request (dequantised pages)
     for r in (0, 3):
