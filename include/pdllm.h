@@ -143,7 +143,8 @@ typedef struct pdllm_attn_desc {
   int64_t slot_table_stride; /* int32 entries per request, >= pdllm_attn_slot_table_stride() */
   /* 0 = choose; >0 = every workgroup takes this many consecutive 64-key tiles of the line formed
    * by the tiles of all (request, KV head, row group) columns, so a workgroup may finish one column
-   * and start the next; columns cut into pieces are merged from fp32 partials in the workspace.
+   * and start the next; columns cut into pieces are merged from partial rows in the workspace (accumulated in
+   * fp32, stored as fp16 with a power-of-two scale per 32 columns: 2^-12 .. 2^-11 of a block's largest element).
    * Overrides num_splits. */
   int32_t tiles_per_workgroup;
   /* optional, pdllm_sparse_decode_attn only: [n_tokens] cache slots (page * page_size + offset) of the active

@@ -14,7 +14,7 @@ import torch
 
 ABS_TOL_BF16 = 2e-2    # max-abs bound of bf16 attention outputs
 REL_TOL_BF16 = 2e-2    # the same bound relative to the largest reference value
-REL_TOL_FP32 = 1e-3    # fp32 partial results, before the rounding of the output to bf16
+REL_TOL_FP32 = 1e-3    # partial results (fp32 accumulation), before the rounding of the output to bf16
 
 
 def bf16_ulp(x: float) -> float:

@@ -41,8 +41,9 @@ struct AttnKParams {
   const int* slot_table;  // [n_req, slot_stride]: cache slot of every visible prefix key; last entry = key count
   long slot_stride;
   const uint8_t* mask;
-  float* ws_o;
-  float* ws_lse;
+  uint16_t* ws_o;    // partial rows, fp16 with one power-of-two scale per 32 columns (store_partial_block)
+  float* ws_lse;     // log-sum-exp of a partial row, log2 units
+  float* ws_scale;   // [row][4] scales of the partial rows
   long q_stride, kn_stride, vn_stride, o_stride;
   long cache_page_stride, cache_token_stride, cache_head_stride;
   long mask_stride;
@@ -87,6 +88,44 @@ __device__ __forceinline__ float half_swap_sum(float x) {
   const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+// Partial results of a column that is cut into pieces: a row of 128 normalised values is stored as fp16 with one
+// power-of-two scale per block of 32 columns -- half the bytes of fp32, rounded (to nearest) at 2^-12 .. 2^-11 of the
+// block's largest element, whatever the magnitude of V.  A lane pair (l, l ^ 32) holds the 32 columns of a block: `o`
+// are this lane's 16 values (columns 32 db + 8 i + 4 he + 0..3 for i = 0..3), inv = 1 / (sum of the row's weights).
+// The block's largest |value| is scaled into [2^14, 2^15).
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store_partial_block(uint16_t* row16, float* scale4, int db, int he, const f32x16& o,
+                                                    float inv) {
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(o[i]));
+  amax = half_swap_max(amax) * inv;
+  unsigned ef = (__float_as_uint(amax) >> 23) & 0xffu;  // biased exponent of the largest element
+  ef = ef < 15u ? 15u : (ef > 254u ? 254u : ef);
+  const float up = __uint_as_float((268u - ef) << 23);  // 2^(14 - E)
+  // this lane's values as packed fp16: word 2 i + k = columns 8 i + 4 he + 2 k, + 1
+  unsigned w[8];
+#pragma unroll
+  for (int i4 = 0; i4 < 4; ++i4) {
+    const f16x2 a = {(_Float16)(o[4 * i4 + 0] * inv * up), (_Float16)(o[4 * i4 + 1] * inv * up)};
+    const f16x2 b = {(_Float16)(o[4 * i4 + 2] * inv * up), (_Float16)(o[4 * i4 + 3] * inv * up)};
+    w[2 * i4] = __builtin_bit_cast(unsigned, a);
+    w[2 * i4 + 1] = __builtin_bit_cast(unsigned, b);
+  }
+  // Of the 16 columns 16 j .. 16 j + 15 the lower lane holds 0-3 and 8-11, the upper one 4-7 and 12-15: after
+  // exchanging the lower lane's second group with the upper lane's first, each lane stores 16 contiguous bytes
+  // (the cost of these stores is their number, not their bytes).
+  uint16_t* wp = row16 + 32 * db + 8 * he;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const auto x = __builtin_amdgcn_permlane32_swap(w[4 * j], w[4 * j + 2], false, false);
+    const auto y = __builtin_amdgcn_permlane32_swap(w[4 * j + 1], w[4 * j + 3], false, false);
+    const uint4 q = {x[0], y[0], x[1], y[1]};
+    *reinterpret_cast<uint4*>(wp + 16 * j) = q;
+  }
+  if (he == 0) scale4[db] = __uint_as_float((ef - 14u) << 23);  // 2^(E - 14)
+}
+
 // Position swizzle of the 16 chunks (16 bytes each) of a 256-byte row: chunk c of row r sits at c ^ swz(r).  Any
 // bijection of the low four row bits keeps the 128-bit K reads (16 consecutive rows, one chunk) and the copies
 // (whole rows) free of bank conflicts.  The transposing 64-bit V reads touch, per group of 32 lanes, four rows

@@ -894,12 +894,7 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
       }
     } else {
       const long R = ((long)(q0 + tq) * p.Hq + kvh * G + g) * p.max_pieces + piece;
-      float* wp = p.ws_o + R * kD + 32 * db + 4 * he;
-#pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        float4 w = {o[4 * i4 + 0] * inv, o[4 * i4 + 1] * inv, o[4 * i4 + 2] * inv, o[4 * i4 + 3] * inv};
-        *reinterpret_cast<float4*>(wp + 8 * i4) = w;
-      }
+      store_partial_block(p.ws_o + R * kD, p.ws_scale + R * 4, db, he, o, inv);
       if (db == 0 && he == 0) p.ws_lse[R] = lfin > 0.f ? mfin + __log2f(lfin) : -INFINITY;  // log2 domain
     }
   };
@@ -1062,8 +1057,9 @@ __global__ __launch_bounds__(256) void attn_slot_table_kernel(const AttnKParams 
 // Reduce the partial results of the columns that were cut into several pieces: one wave per
 // (token, q-head) row.  Rows of a column with a single piece were written directly.
 struct MergeParams {
-  const float* ws_o;
+  const uint16_t* ws_o;  // fp16 partial rows, see store_partial_block
   const float* ws_lse;
+  const float* ws_scale;
   __bf16* out;
   const int* q_start_loc;
   long o_stride, n_tokens;
@@ -1095,9 +1091,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const MergeParams m) {
     m.v_cache[slot * cpr + ch] = vv;
     return;
   }
-  // 32 lanes per row (4 columns each), 8 rows per workgroup
-  const int l = threadIdx.x & 31;
-  const long row = (long)((int)blockIdx.x - m.store_blocks) * 8 + (threadIdx.x >> 5);
+  // 16 lanes per row (8 columns = 16 bytes of a partial row each), 16 rows per workgroup
+  const int l = threadIdx.x & 15;
+  const long row = (long)((int)blockIdx.x - m.store_blocks) * 16 + (threadIdx.x >> 4);
   const long per_req = (long)m.max_q_len * m.Hq;
   if (row >= per_req * m.n_req) return;
   const int req = (int)(row / per_req);
@@ -1120,36 +1116,47 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const MergeParams m) {
   // folded into the running maximum.  A piece without keys has lse = -inf and weight 0; what its row holds is
   // never used.
   float M = -INFINITY, L = 0.f;
-  float4 acc = {0.f, 0.f, 0.f, 0.f};
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int s0 = 0; s0 < np; s0 += 4) {
-    float lse[4];
-    float4 o[4];
+    float lse[4], sc[4];
+    uint4 o[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const bool on = s0 + u < np;
       lse[u] = on ? m.ws_lse[R + s0 + u] : -INFINITY;
-      o[u] = on ? *reinterpret_cast<const float4*>(m.ws_o + (R + s0 + u) * kD + 4 * l) : float4{0.f, 0.f, 0.f, 0.f};
+      sc[u] = on ? m.ws_scale[(R + s0 + u) * 4 + (l >> 2)] : 0.f;
+      o[u] = on ? *reinterpret_cast<const uint4*>(m.ws_o + (R + s0 + u) * kD + 8 * l) : uint4{0u, 0u, 0u, 0u};
     }
     const float Mn = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
     if (Mn == -INFINITY) continue;
     const float r = M == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(M - Mn);
-    acc.x *= r; acc.y *= r; acc.z *= r; acc.w *= r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= r;
     L *= r;
     M = Mn;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const float w = lse[u] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(lse[u] - M);
       if (w > 0.f) {
-        acc.x += w * o[u].x; acc.y += w * o[u].y; acc.z += w * o[u].z; acc.w += w * o[u].w;
+        const unsigned words[4] = {o[u].x, o[u].y, o[u].z, o[u].w};
+        const float ws = w * sc[u];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const f16x2 h2 = __builtin_bit_cast(f16x2, words[e]);
+          acc[2 * e] += ws * (float)h2[0];
+          acc[2 * e + 1] += ws * (float)h2[1];
+        }
         L += w;
       }
     }
   }
   const float inv = L > 0.f ? 1.f / L : 0.f;
-  uint2 packed;
-  packed.x = pack_bf16x2(acc.x * inv, acc.y * inv);
-  packed.y = pack_bf16x2(acc.z * inv, acc.w * inv);
-  *reinterpret_cast<uint2*>(m.out + (long)(q0 + tq) * m.o_stride + (long)head * kD + 4 * l) = packed;
+  uint4 packed;
+  packed.x = pack_bf16x2(acc[0] * inv, acc[1] * inv);
+  packed.y = pack_bf16x2(acc[2] * inv, acc[3] * inv);
+  packed.z = pack_bf16x2(acc[4] * inv, acc[5] * inv);
+  packed.w = pack_bf16x2(acc[6] * inv, acc[7] * inv);
+  *reinterpret_cast<uint4*>(m.out + (long)(q0 + tq) * m.o_stride + (long)head * kD + 8 * l) = packed;
 }
 
 // ---------------------------------------------------------------------------
@@ -1252,7 +1259,7 @@ static int dyn_lds_bytes(int J, int mask_mode) {
 // All tiles of all columns (request, KV head, row group) lie on one line of n_cols * t_lin
 // positions; workgroup g takes positions [g * span, (g + 1) * span).  span = t_lin gives one
 // workgroup per column; a smaller span that does not divide t_lin lets pieces of two columns
-// share a workgroup, which balances any shape over the CUs at the price of fp32 partials.
+// share a workgroup, which balances any shape over the CUs at the price of partial rows in the workspace.
 // Unit of time: one wave doing one 32-row block of one 64-key tile on a CU of its own.  A
 // workgroup alone on a CU spends (fixed + blocks per wave) per tile; two workgroups sharing a CU
 // (at most 4 row blocks, LDS footprint <= 80 KB) overlap matrix and vector work and take kPair of the
@@ -1358,7 +1365,8 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
       }
       double cost = serial * ((double)span * (kFixed + upw[ji]) + kPiece * (cut && t_lin % span ? 2.0 : 1.0)) + 1.0;
       if (cut) {
-        // fp32 partials written and read back (~4 MB per unit of time), plus the merge launch
+        // partials written and read back, plus the merge launch (the constants were fitted when a partial row was
+        // 516 bytes of fp32; it is 276 bytes now and the fit was left as it is: the plans it picks are still the best)
         const double avg_pieces = (double)t_lin / (double)span + (t_lin % span ? 1.0 : 0.0);
         const double part_bytes = (double)units * rows * avg_pieces * (kD + 1) * 4.0 * 2.0;
         cost += part_bytes / 4.0e6 + 4.0;
@@ -1394,7 +1402,7 @@ static bool needs_own_table(const pdllm_attn_desc* d, bool prefill) {
 static int64_t partial_bytes_for(const pdllm_attn_desc* d, int max_pieces) {
   if (max_pieces <= 1) return 0;
   const int64_t rows = d->n_tokens * d->num_q_heads;
-  return rows * max_pieces * (int64_t)(kD + 1) * 4;
+  return rows * max_pieces * (int64_t)(kD * 2 + 4 + 16);  // fp16 row, log-sum-exp, four scales
 }
 static int64_t ws_bytes_for(const pdllm_attn_desc* d, int max_pieces, bool prefill) {
   int64_t b = partial_bytes_for(d, max_pieces);
@@ -1442,8 +1450,9 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
   p.q_start_loc = d->q_start_loc;
   p.mask = d->mask_mode == PDLLM_MASK_DENSE ? d->mask : nullptr;
   const int64_t rows = d->n_tokens * d->num_q_heads;
-  p.ws_o = plan.max_pieces > 1 ? static_cast<float*>(d->workspace) : nullptr;
-  p.ws_lse = p.ws_o ? p.ws_o + rows * plan.max_pieces * kD : nullptr;
+  p.ws_o = plan.max_pieces > 1 ? static_cast<uint16_t*>(d->workspace) : nullptr;
+  p.ws_lse = p.ws_o ? reinterpret_cast<float*>(p.ws_o + rows * plan.max_pieces * kD) : nullptr;
+  p.ws_scale = p.ws_o ? p.ws_lse + rows * plan.max_pieces : nullptr;
   if (has_cache) {
     fill_table_params(d, p);
     p.slot_stride = d->slot_table ? d->slot_table_stride : slot_table_stride_for(d);
@@ -1534,13 +1543,13 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
   }
   if (plan.max_pieces > 1) {
     MergeParams m = {};
-    m.ws_o = p.ws_o; m.ws_lse = p.ws_lse; m.out = p.out; m.q_start_loc = p.q_start_loc;
+    m.ws_o = p.ws_o; m.ws_lse = p.ws_lse; m.ws_scale = p.ws_scale; m.out = p.out; m.q_start_loc = p.q_start_loc;
     m.o_stride = p.o_stride; m.n_tokens = p.n_tokens;
     m.n_req = p.n_req; m.max_q_len = p.max_q_len; m.Hq = p.Hq; m.Hkv = p.Hkv;
     m.rows_per_group = 32 * plan.J; m.row_tiles = plan.row_tiles; m.reversed = p.mask_mode == PDLLM_MASK_CAUSAL;
     m.t_lin = plan.t_lin; m.span = plan.span; m.max_pieces = plan.max_pieces; m.head = plan.head;
     const long mrows = (long)d->n_req * d->max_q_len * d->num_q_heads;
-    const int merge_blocks = (int)((mrows + 7) / 8);
+    const int merge_blocks = (int)((mrows + 15) / 16);  // 16 rows per workgroup
     if (store_in_merge) {
       m.store_slots = d->active_slot_mapping;
       m.k_new = static_cast<const uint4*>(d->k_new);

@@ -700,12 +700,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd2_kernel(const AttnKParams
       const int g = rix - tq * G;
       const float inv = lfin > 0.f ? 1.f / lfin : 0.f;
       const long R = ((long)(q0 + tq) * p.Hq + kvh * G + g) * p.max_pieces + piece;
-      float* wp = p.ws_o + R * kD + 32 * db + 4 * he;
-#pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        float4 w = {o[4 * i4 + 0] * inv, o[4 * i4 + 1] * inv, o[4 * i4 + 2] * inv, o[4 * i4 + 3] * inv};
-        *reinterpret_cast<float4*>(wp + 8 * i4) = w;
-      }
+      store_partial_block(p.ws_o + R * kD, p.ws_scale + R * 4, db, he, o, inv);
       if (db == 0 && he == 0) p.ws_lse[R] = lfin > 0.f ? mfin + __log2f(lfin) : -INFINITY;  // log2 domain
     };
     // rows of an uncut column go through an 8 KB strip of the (now free) K ring per wave, 64 columns at a time,
