@@ -195,7 +195,8 @@ int pdllm_attn_plan(const pdllm_attn_desc* desc, int32_t prefill, int32_t* rows_
                     int32_t* num_splits);
 
 /* The same plan as one line of text ("<kernel> kv=<dtype> row_blocks=J grid=.. span=.. head=.. set=.. tiles=..
- * pieces=.."): which kernel runs and how the tiles of the launch are cut over workgroups.  No counterpart in the
+ * pieces=.. partial_row_bytes=.."): which kernel runs, how the tiles of the launch are cut over workgroups and how
+ * many bytes a partial row of a cut column takes in the workspace.  No counterpart in the
  * reference; it identifies a launch configuration so that measurements (profiles, counters) can be matched to the
  * configuration they were taken on.  text receives at most text_bytes bytes including the terminating 0. */
 int pdllm_attn_plan_describe(const pdllm_attn_desc* desc, int32_t prefill, char* text, int32_t text_bytes);

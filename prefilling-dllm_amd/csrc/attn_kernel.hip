@@ -1630,9 +1630,11 @@ extern "C" int pdllm_attn_plan_describe(const pdllm_attn_desc* desc, int32_t pre
   const pdllm::AttnPlan plan = pdllm::make_plan(desc, prefill != 0);
   const bool fp8 = !prefill && desc->k_cache != nullptr && desc->max_ctx_len > 0 && desc->kv_dtype == PDLLM_KV_FP8_E4M3;
   const char* kernel = plan.J == 8 && !fp8 ? "attn_fwd2_kernel" : "attn_fwd_kernel";
-  const int n = snprintf(text, (size_t)text_bytes, "%s kv=%s row_blocks=%d grid=%d span=%d head=%d set=%d tiles=%d pieces=%d",
+  // (the bytes of a partial row are part of the text: traffic figures taken for one format do not describe another)
+  const int n = snprintf(text, (size_t)text_bytes,
+                         "%s kv=%s row_blocks=%d grid=%d span=%d head=%d set=%d tiles=%d pieces=%d partial_row_bytes=%d",
                          kernel, fp8 ? "fp8" : "bf16", plan.J, plan.grid, plan.span, plan.head, plan.wg_set,
-                         plan.t_lin, plan.max_pieces);
+                         plan.t_lin, plan.max_pieces, plan.max_pieces > 1 ? pdllm::kD * 2 + 4 + 16 : 0);
   return n > 0 && n < text_bytes ? PDLLM_OK : PDLLM_ERR_SHAPE;
 }
 
