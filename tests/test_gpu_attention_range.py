@@ -165,3 +165,34 @@ def test_fp32_partials_before_bf16_rounding(dev, splits, rows):
     # the bf16 output of the same launch is the merged result rounded
     assert_attn_close(out, ref.float(), f"{splits} splits")
     assert float((out.double() - merged).abs().max()) <= 2.0 ** -8 * float(ref.abs().max()) * 1.01
+
+
+@pytest.mark.parametrize("plan", [dict(rows_per_group=128, num_splits=3), dict(rows_per_group=256, num_splits=2),
+                                  dict(rows_per_group=32, num_splits=4), dict(rows_per_group=128, tiles_per_workgroup=5),
+                                  dict()],
+                         ids=lambda p: "-".join(f"{k[0]}{v}" for k, v in p.items()) or "default")
+@pytest.mark.parametrize("shift", [100, -60, 17, -33])
+def test_values_scaled_by_a_power_of_two_scale_the_output_exactly(dev, plan, shift):
+    """V * 2^k gives out * 2^k bit for bit: every product and sum of the kernel scales exactly, and the partial rows
+    of a cut column (fp16 with a power-of-two scale per 32 columns) must follow the magnitude of V whatever it is --
+    values of 1e29 and of 1e-19 alike.  (Far below 2^-60 single products leave the normal range of fp32 and the
+    scaling stops being exact.)"""
+    case = configs.chunked_prefix_case(71, n_req=2, n_chunks=4, chunk_tokens=512, topk=3, q_len=40,
+                                       shared_prefix=False)
+    base = _run(case, dev, **plan)
+    f = 2.0 ** shift
+    case.v_cache = (case.v_cache.float() * f).to(torch.bfloat16)
+    case.v_new = (case.v_new.float() * f).to(torch.bfloat16)
+    assert torch.isfinite(case.v_cache.float()).all() and float(case.v_cache.float().abs().max()) > 0
+    scaled = _run(case, dev, **plan)
+    assert torch.isfinite(scaled).all()
+    assert torch.equal(scaled, base * f), float((scaled / f - base).abs().max())
+    assert_attn_close(scaled / f, _oracle(_unscaled(case, f)), f"V * 2^{shift}")
+
+
+def _unscaled(case, f):
+    import copy
+    c = copy.copy(case)
+    c.v_cache = (case.v_cache.float() / f).to(torch.bfloat16)
+    c.v_new = (case.v_new.float() / f).to(torch.bfloat16)
+    return c
