@@ -1365,10 +1365,9 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
       }
       double cost = serial * ((double)span * (kFixed + upw[ji]) + kPiece * (cut && t_lin % span ? 2.0 : 1.0)) + 1.0;
       if (cut) {
-        // partials written and read back, plus the merge launch (the constants were fitted when a partial row was
-        // 516 bytes of fp32; it is 276 bytes now and the fit was left as it is: the plans it picks are still the best)
+        // partial rows written and read back (~4 MB per unit of time), plus the merge launch
         const double avg_pieces = (double)t_lin / (double)span + (t_lin % span ? 1.0 : 0.0);
-        const double part_bytes = (double)units * rows * avg_pieces * (kD + 1) * 4.0 * 2.0;
+        const double part_bytes = (double)units * rows * avg_pieces * (kD * 2 + 4 + 16) * 2.0;
         cost += part_bytes / 4.0e6 + 4.0;
       }
       if (head > 0) cost *= 0.97;  // the set's workgroups share their tiles in L2: less traffic for the same cut
