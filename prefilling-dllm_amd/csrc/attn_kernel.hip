@@ -1287,7 +1287,9 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   const long units = (long)d->n_req * d->num_kv_heads;
   const bool fp8 = !prefill && d->k_cache != nullptr && d->max_ctx_len > 0 && d->kv_dtype == PDLLM_KV_FP8_E4M3;
   const int cus = compute_units();
-  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 1.5, kWide = 1.25;
+  // kPiece: what a piece costs outside its tile loop (three round trips to memory before the first MFMA, the
+  // last PV, the partial rows): about 3.2 tiles of a 4-wave workgroup
+  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 4.3, kWide = 1.25;
   constexpr int kStaticLds = 66 * 1024;
   static const int js[] = {1, 2, 4, 5, 6, 8};
   static const double upw[] = {0.45, 0.75, 1.0, 1.25, 1.5, 1.0};
@@ -1309,6 +1311,7 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
     // candidate spans: whole columns, columns cut into 2..16 equal parts, and the balanced cut
     for (int cand = 0; cand <= 20; ++cand) {
       long t_lin = T, span, head = 0, wg_set = 0;
+      double set_load = 0.0;
       if (cand == 0) {
         span = T;
       } else if (cand <= 15) {
@@ -1333,12 +1336,32 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
         if (prefill || row_tiles < 2) continue;
         const long k = (cand == 19 ? slots : 2 * slots) / units;
         if (k <= row_tiles) continue;
-        // a head workgroup handles one piece, the others two or three: it takes kHeadExtra tiles more
-        constexpr long kHeadExtra = 3;
-        span = (row_tiles * (T - kHeadExtra) + k - 1) / k;
-        head = span + kHeadExtra;
-        if (head >= T || span < 4) continue;
+        // A head workgroup handles one piece of `head` tiles; the others cut the rest of the set's columns into
+        // spans and handle two or three pieces each.  The head is made `extra` tiles longer than a span; which
+        // `extra` gives the shortest longest workgroup depends on where the cuts fall in the columns (a cut that
+        // coincides with the end of a column saves a piece), so the candidates are laid out and compared.
+        const double tile_cost = kFixed + upw[ji], piece_cost = kPiece;
+        double best_load = 1e300;
+        long best_span = 0, best_head = 0;
+        for (long extra = 0; extra <= 12; ++extra) {
+          const long sp = (row_tiles * (T - extra) + k - 1) / k;
+          const long hd = sp + extra;
+          if (hd >= T || sp < 4) continue;
+          const long tail_len = T - hd, tail_total = row_tiles * tail_len;
+          double load = (double)hd * tile_cost + piece_cost;
+          for (long a = 0; a < tail_total; a += sp) {
+            const long b = a + sp < tail_total ? a + sp : tail_total;
+            const long n_pieces = (b - 1) / tail_len - a / tail_len + 1;
+            const double l = (double)(b - a) * tile_cost + piece_cost * (double)n_pieces;
+            load = l > load ? l : load;
+          }
+          if (load < best_load) { best_load = load; best_span = sp; best_head = hd; }
+        }
+        if (best_span == 0) continue;
+        span = best_span;
+        head = best_head;
         wg_set = k;
+        set_load = best_load;
       }
       if (d->tiles_per_workgroup > 0) {
         if (cand != 18) continue;
@@ -1363,7 +1386,10 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
           pieces = np > pieces ? np : pieces;
         }
       }
-      double cost = serial * ((double)span * (kFixed + upw[ji]) + kPiece * (cut && t_lin % span ? 2.0 : 1.0)) + 1.0;
+      // the most loaded workgroup: its tiles and its pieces (two where the cuts do not respect the columns)
+      const double wg_load = head > 0 ? set_load
+                                      : (double)span * (kFixed + upw[ji]) + kPiece * (cut && t_lin % span ? 2.0 : 1.0);
+      double cost = serial * wg_load + 1.0;
       if (cut) {
         // partial rows written and read back (~4 MB per unit of time), plus the merge launch
         const double avg_pieces = (double)t_lin / (double)span + (t_lin % span ? 1.0 : 0.0);
