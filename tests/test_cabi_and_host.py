@@ -98,6 +98,62 @@ def test_attention_plan_is_host_only():
     assert ops.attention_plan(8, 28, 4, max_q_len=160, max_ctx_len=4096, rows_per_group=128, num_splits=2) == (128, 2)
 
 
+def _decode_desc(n_req, q_len, ctx, hq=28, hkv=4, fp8=False):
+    """A decode descriptor over a paged cache with made-up (non-NULL, aligned) addresses: the planner and the
+    validation only read sizes and strides."""
+    import torch
+    from prefilling_dllm_amd import _lib
+    dummy = torch.empty(64, dtype=torch.int32)
+    a = (dummy.data_ptr() + 15) & ~15
+    d = _lib.AttnDesc()
+    for f in ("q", "k_new", "v_new", "out", "q_start_loc", "k_cache", "v_cache", "block_table", "range_ptr",
+              "range_start", "range_len"):
+        setattr(d, f, a)
+    if fp8:
+        d.k_scale = d.v_scale = a
+    d.q_stride = d.o_stride = hq * 128
+    d.kn_stride = d.vn_stride = hkv * 128
+    d.cache_head_stride, d.cache_token_stride, d.cache_page_stride = 128, hkv * 128, 256 * hkv * 128
+    d.n_tokens, d.n_pages, d.bt_stride, d.page_size = n_req * q_len, 4096, 1024, 256
+    d.n_req, d.max_q_len, d.max_ctx_len, d.max_ranges = n_req, q_len, ctx, 16
+    d.num_q_heads, d.num_kv_heads, d.head_dim = hq, hkv, 128
+    d.kv_dtype = _lib.KV_FP8_E4M3 if fp8 else _lib.KV_BF16
+    d.sm_scale = 128 ** -0.5
+    return d
+
+
+def _plan_text(desc):
+    from prefilling_dllm_amd import _lib
+    buf = ctypes.create_string_buffer(256)
+    _lib.check(_lib.lib.pdllm_attn_plan_describe(ctypes.byref(desc), 0, buf, 256), "plan")
+    return dict(kv.split("=") for kv in buf.value.decode().split()[1:]), buf.value.decode().split()[0]
+
+
+def test_planner_lays_out_the_set_cut_without_a_gpu():
+    """The cut of the benchmark's decode step (8 requests x 160 rows x 7 heads per KV head over 4096 + 160 keys, 256
+    compute units assumed without a device): 16 workgroups per (request, KV head), nine of them on the leading 40
+    tiles of one row group each, the other seven on spans of 36 tiles of the nine tails of 27 -- every third cut
+    falls on the end of a column, so no workgroup has more than two pieces and no row more than three."""
+    f, kernel = _plan_text(_decode_desc(8, 160, 4096))
+    assert kernel == "attn_fwd_kernel" and f["kv"] == "bf16" and f["row_blocks"] == "4"
+    assert (f["grid"], f["set"], f["head"], f["span"], f["tiles"], f["pieces"]) == ("512", "16", "40", "36", "67", "3")
+    assert f["partial_row_bytes"] == "276"
+    head, span, tiles, rt, k = 40, 36, 67, 9, 16
+    tail = tiles - head
+    loads = [(min(a + span, rt * tail) - a, (min(a + span, rt * tail) - 1) // tail - a // tail + 1)
+             for a in range(0, rt * tail, span)]
+    assert len(loads) == k - rt and max(p for _, p in loads) == 2 and sum(p for _, p in loads) == 13
+    # 32 response rows only: the eight-wave kernel, every (request, KV head) cut into eight aligned pieces
+    f, kernel = _plan_text(_decode_desc(8, 32, 4096))
+    assert kernel == "attn_fwd2_kernel" and (f["row_blocks"], f["grid"], f["span"], f["head"]) == ("8", "256", "9", "0")
+    # fp8 pages, 160 rows per head: one group of five row blocks, two aligned pieces
+    f, kernel = _plan_text(_decode_desc(4, 160, 16 * 1025, hq=32, hkv=32, fp8=True))
+    assert kernel == "attn_fwd_kernel" and (f["kv"], f["row_blocks"], f["grid"], f["pieces"]) == ("fp8", "5", "256", "2")
+    # one workgroup per column when the columns fill the chip: no partial rows
+    f, _ = _plan_text(_decode_desc(64, 128, 1024))
+    assert f["pieces"] == "1" and f["partial_row_bytes"] == "0"
+
+
 def test_page_pool_semantics():
     """What callers of the reference's allocator observe (fastdllm_engine.py:88-167): pages are handed out in the
     order they became free, refcounts, the exhaustion error, hash-keyed prefix reuse and eviction."""
