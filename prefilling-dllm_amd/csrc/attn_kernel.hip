@@ -344,9 +344,14 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
 #pragma unroll
     for (int i = 0; i < kDmaGroups; ++i) nslot[i] = tbl[t * kKT + 4 * NW * i + lane_row];
   };
+  // (rows past the active block -- a ragged last tile, or a tile past the end of the piece that is copied
+  // but never read -- repeat the last row: always a valid address)
   auto load_slots_new = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < kDmaGroups; ++i) nslot[i] = (t - Tc) * kKT + 4 * NW * i + lane_row;
+    for (int i = 0; i < kDmaGroups; ++i) {
+      const int a = (t - Tc) * kKT + 4 * NW * i + lane_row;
+      nslot[i] = a < Sa ? a : Sa - 1;
+    }
   };
   auto load_slots = [&](int t) __attribute__((always_inline)) {
     if (t < Tc) {
@@ -834,15 +839,17 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
       __syncthreads();
       {
         using Generic = std::integral_constant<int, 0>;
+        // The steady forms need a tile t that is whole and unmasked and a tile t + 1 inside the piece.  Their copies
+        // (V(t+1), K(t+2)) and slots (t+3) are issued unconditionally: past the end of the piece they land in free
+        // buffers and are never read, but they must come from the tensor the form assumes -- prefix tiles up to
+        // t + 3 for the first form (table entries exist for whole_ctx tiles), clamped rows for the second.
         const int whole_ctx = ctx_total / kKT;  // tiles of the prefix without a ragged end
-        const int ctx_end = (T1 < whole_ctx ? T1 : whole_ctx) - 3;
+        const int ctx_end = T1 - 1 < whole_ctx - 3 ? T1 - 1 : whole_ctx - 3;
         // active tiles that are whole and visible to every row of this row group
         int open_tiles = Sa / kKT;
         if (p.mask_mode == PDLLM_MASK_CAUSAL) open_tiles = (tq_first + 1) / kKT < open_tiles ? (tq_first + 1) / kKT : open_tiles;
         if (p.mask_mode == PDLLM_MASK_DENSE) open_tiles = 0;
-        int new_end = Tc + Sa / kKT - 3;
-        new_end = new_end < T1 - 3 ? new_end : T1 - 3;
-        new_end = new_end < Tc + open_tiles ? new_end : Tc + open_tiles;
+        const int new_end = T1 - 1 < Tc + open_tiles ? T1 - 1 : Tc + open_tiles;
         int t = T0;
         if constexpr (BUF) {  // (the wide-address form keeps the one general loop: it has no registers to spare)
           for (; t < ctx_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 1>{});
