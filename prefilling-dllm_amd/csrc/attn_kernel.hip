@@ -1401,7 +1401,7 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
         // partial rows written and read back (~4 MB per unit of time), plus the merge launch
         const double avg_pieces = (double)t_lin / (double)span + (t_lin % span ? 1.0 : 0.0);
         const double part_bytes = (double)units * rows * avg_pieces * (kD * 2 + 4 + 16) * 2.0;
-        cost += part_bytes / 4.0e6 + 4.0;
+        cost += part_bytes / 4.0e6 + 4.0 + 0.3 * avg_pieces;  // (the merge folds a row's pieces one after the other)
       }
       if (head > 0) cost *= 0.97;  // the set's workgroups share their tiles in L2: less traffic for the same cut
       if (cost < best_cost) {
