@@ -169,7 +169,7 @@ template <int N, typename T>
 __device__ __forceinline__ void lds_wait(T& x) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N) : "memory");
 }
-// the same, and also a fence for three values of the vector pipeline: work that produces them
+// the same, and also a fence for two values of the vector pipeline: work that produces them
 // stays before this point, work that consumes them after it (pins the interleaving of softmax
 // arithmetic with the MFMAs, which the compiler would otherwise gather in one place)
 // `keep` is only named as an input: it holds the fragment the MFMA of the step before is still
@@ -177,12 +177,17 @@ __device__ __forceinline__ void lds_wait(T& x) {
 // vector instructions in between (a write to a source of a running MFMA stalls the wave until
 // the MFMA has finished, which would serialise the two pipelines).
 template <int N, typename T>
-__device__ __forceinline__ void lds_wait_pin(T& x, float& a, float& b, float& c, const T& keep) {
-  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(x), "+v"(a), "+v"(b), "+v"(c) : "n"(N), "v"(keep) : "memory");
+__device__ __forceinline__ void lds_wait_pin(T& x, float& a, float& b, const T& keep) {
+  asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(x), "+v"(a), "+v"(b) : "n"(N), "v"(keep) : "memory");
 }
 template <int N, typename T>
 __device__ __forceinline__ void lds_wait2(T& x, T& y) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N) : "memory");
+}
+// the same, and a fence for one value of the vector pipeline (see lds_wait_pin)
+template <int N, typename T>
+__device__ __forceinline__ void lds_wait2_pin(T& x, T& y, float& a) {
+  asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(x), "+v"(y), "+v"(a) : "n"(N) : "memory");
 }
 
 }  // namespace pdllm

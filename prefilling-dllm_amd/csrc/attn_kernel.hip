@@ -340,9 +340,13 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
   const unsigned vn_row16 = (unsigned)((p.vn_stride * 2) >> 4);
   int nslot[kDmaGroups];
   // the same for a tile known to be a whole tile of the prefix / of the active block
+  // (uniform 64-bit base + 32-bit lane offset + immediate: no vector address arithmetic per tile)
+  const unsigned lane_row_b = (unsigned)lane_row * 4u;
   auto load_slots_ctx = [&](int t) __attribute__((always_inline)) {
+    const char* tile_tbl = reinterpret_cast<const char*>(tbl + (long)t * kKT);
 #pragma unroll
-    for (int i = 0; i < kDmaGroups; ++i) nslot[i] = tbl[t * kKT + 4 * NW * i + lane_row];
+    for (int i = 0; i < kDmaGroups; ++i)
+      nslot[i] = *reinterpret_cast<const int*>(tile_tbl + (unsigned long)lane_row_b + 16 * NW * i);
   };
   // (rows past the active block -- a ragged last tile, or a tile past the end of the piece that is copied
   // but never read -- repeat the last row: always a valid address)
@@ -585,7 +589,11 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
       // offset per lane from one 24-bit multiply-add) costs the issuing wave about 15 clk, the
       // flat-address form 60 and more.
       const unsigned lane_b16 = (unsigned)lane_ch << 4;
-      auto copy_row = [&](const char* base, unsigned row16, int slot, char* dst) __attribute__((always_inline)) {
+      // LDS address of this wave's part of buffer 0; made opaque once per iteration so that the copy destinations
+      // are one scalar add each (as loop invariants they would be sixteen spilled scalars in the unrolled loops)
+      unsigned wave_lds = lds_base + wave * 1024;
+      auto copy_row = [&](const char* base, unsigned row16, int slot, unsigned dst_off) __attribute__((always_inline)) {
+        auto* dst = (__attribute__((address_space(3))) char*)(size_t)(wave_lds + dst_off);
         if constexpr (BUF) {
           const __amdgpu_buffer_rsrc_t rs =
               __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, 0xffffffff, 0x00020000);
@@ -602,13 +610,13 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
         constexpr int SRC = decltype(src_tag)::value;
         const bool ctx = SRC == 1 || (SRC == 0 && t < Tc);
         copy_row(ctx ? kc_base : kn_base, ctx ? cache_row16 : kn_row16, nslot[i],
-                 lds + buf * kBufBytes + wave * 1024 + i * (NW * 1024));
+                 (unsigned)(buf * kBufBytes + i * (NW * 1024)));
       };
       auto issue_v1 = [&](int t, int buf, int i, auto src_tag) __attribute__((always_inline)) {
         constexpr int SRC = decltype(src_tag)::value;
         const bool ctx = SRC == 1 || (SRC == 0 && t < Tc);
         copy_row(ctx ? vc_base : vn_base, ctx ? cache_row16 : vn_row16, nsv[i],
-                 lds + buf * kBufBytes + kTileBytes + wave * 1024 + i * (NW * 1024));
+                 (unsigned)(buf * kBufBytes + kTileBytes + i * (NW * 1024)));
       };
       auto issue_k = [&](int t, int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -620,12 +628,16 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
       };
       // K fragment read of QK step stp / V^T fragment read of PV step stp; ka and va point into the
       // buffer in use and move to the other one after every tile
-      auto rdk = [&](bf16x8& dst, int stp) __attribute__((always_inline)) {
-        if ((stp >> 3) == 0) lds_read_b128<0>(dst, ka[stp & 7]);
-        else lds_read_b128<32 * kRowBytes>(dst, ka[stp & 7]);
+      // (par_tag: -1 = as described; 0 / 1 = an iteration of known buffer parity in a loop unrolled by two,
+      // where ka and va stay on buffer 0 and the buffer is part of the immediate offset)
+      auto rdkp = [&](bf16x8& dst, int stp, auto par_tag) __attribute__((always_inline)) {
+        constexpr int boff = decltype(par_tag)::value == 0 ? kBufBytes : 0;  // K(t+1) of an even iteration: buffer 1
+        if ((stp >> 3) == 0) lds_read_b128<boff>(dst, ka[stp & 7]);
+        else lds_read_b128<boff + 32 * kRowBytes>(dst, ka[stp & 7]);
       };
-      auto rdv = [&](s16x4& dst, int stp, int r) __attribute__((always_inline)) {
-        constexpr int base = kTileBytes;
+      auto rdk = [&](bf16x8& dst, int stp) __attribute__((always_inline)) { rdkp(dst, stp, std::integral_constant<int, -1>{}); };
+      auto rdv = [&](s16x4& dst, int stp, int r, auto par_tag) __attribute__((always_inline)) {
+        constexpr int base = kTileBytes + (decltype(par_tag)::value == 1 ? kBufBytes : 0);  // V(t) of an odd iteration: buffer 1
         const int db = stp & 3, kj = stp >> 2;
         if (kj == 0) lds_read_tr16_b64<base>(dst, va[r][db]);
         else if (kj == 1) lds_read_tr16_b64<base + 16 * kRowBytes>(dst, va[r][db]);
@@ -644,10 +656,14 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
       // one iteration: softmax of tile t (scores in Sc) interleaved with QK of tile t + 1 (into Sn),
       // then PV of tile t.  PAR = buffer of V(t); K(t+1) sits in the other buffer.
       int flip = kBufBytes;  // ka: buffer 1 -> 0 -> 1 ..., va: buffer 0 -> 1 -> 0 ...
+      float mx_carry = 0.f;  // unmasked row maximum (log2 units) of the scores the next iteration starts with
       // steady (mode 1 / 2): tiles t .. t + 3 are whole tiles of the prefix / of the active block, lie inside this
       // piece, and tile t needs no mask for any row -- every copy comes from one tensor, nothing to mask, no
       // end-of-piece cases (the same code with those decisions made at compile time)
-      auto iter = [&](int t, int PAR, f32x16 (&Sc)[2], auto steady_tag) __attribute__((always_inline)) {
+      auto iter = [&](int t, int par_rt, f32x16 (&Sc)[2], auto steady_tag, auto par_tag) __attribute__((always_inline)) {
+        constexpr int PARC = decltype(par_tag)::value;
+        const int PAR = PARC >= 0 ? PARC : par_rt;
+        asm volatile("" : "+s"(wave_lds));
         constexpr int MODE = decltype(steady_tag)::value;
         constexpr bool STEADY = MODE != 0;
         const bool has_next = STEADY || t + 1 < T1;
@@ -685,12 +701,19 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
             }
           }
         }
-        float mx = fmaxf(Sc[0][0], Sc[0][1]);
+        // A steady tile has no mask: its row maximum was taken from the finished scores during the PV
+        // phase of the iteration before (or the prologue), where the vector unit idles under the MFMAs.
+        float mx;
+        if constexpr (STEADY) {
+          mx = mx_carry;
+        } else {
+          mx = fmaxf(Sc[0][0], Sc[0][1]);
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+          for (int b = 0; b < 2; ++b)
 #pragma unroll
-          for (int i = (b == 0 ? 2 : 0); i < 16; i += 2) mx = fmaxf(fmaxf(mx, Sc[b][i]), Sc[b][i + 1]);
-        mx = half_swap_max(mx) * c;  // log2 units
+            for (int i = (b == 0 ? 2 : 0); i < 16; i += 2) mx = fmaxf(fmaxf(mx, Sc[b][i]), Sc[b][i + 1]);
+          mx = half_swap_max(mx) * c;  // log2 units
+        }
         const bool need = mx > MA + kRescaleSlack;
         if (__builtin_amdgcn_ballot_w64(need) != 0) {
           const float Mn = fmaxf(MA, mx);
@@ -705,7 +728,7 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
           }
         }
         // ---- exponentials of tile t, two per step, between the MFMAs of QK(t+1) ----
-        const float negM = (MA == -INFINITY) ? 0.f : -MA;
+        float negM = (MA == -INFINITY) ? 0.f : -MA;
         f32x16 Sn[2];
 #pragma unroll
         for (int b = 0; b < 2; ++b)
@@ -725,24 +748,22 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
         if (has_next) {
           bf16x8 kf[PF];
 #pragma unroll
-          for (int i = 0; i < PF; ++i) rdk(kf[i], i);
+          for (int i = 0; i < PF; ++i) rdkp(kf[i], i, par_tag);
           bf16x8 used = kf[0];  // fragment of the MFMA issued in the step before
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int stp = 0; stp < NS; ++stp) {
             {
-              // wait for this step's K fragment; the step's two scores enter and the running sum of
-              // the step before leaves through the same statement
-              float e0 = Sc[stp >> 3][2 * (stp & 7)];
-              float e1 = Sc[stp >> 3][2 * (stp & 7) + 1];
+              // wait for this step's K fragment; the subtrahend of the step's exponentials and the running
+              // sum of the step before pass through the same statement: the step's arithmetic stays behind
+              // the wait, the arithmetic of the step before in front of it.  (The scores themselves do not
+              // pass through it: a tied operand that is one element of a 16-register tuple costs a move.)
               const int young = NS - 1 - stp < PF - 1 ? NS - 1 - stp : PF - 1;
-              if (young == 3) lds_wait_pin<3>(kf[stp % PF], e0, e1, psum, used);
-              else if (young == 2) lds_wait_pin<2>(kf[stp % PF], e0, e1, psum, used);
-              else if (young == 1) lds_wait_pin<1>(kf[stp % PF], e0, e1, psum, used);
-              else lds_wait_pin<0>(kf[stp % PF], e0, e1, psum, used);
+              if (young == 3) lds_wait_pin<3>(kf[stp % PF], negM, psum, used);
+              else if (young == 2) lds_wait_pin<2>(kf[stp % PF], negM, psum, used);
+              else if (young == 1) lds_wait_pin<1>(kf[stp % PF], negM, psum, used);
+              else lds_wait_pin<0>(kf[stp % PF], negM, psum, used);
               used = kf[stp % PF];
-              Sc[stp >> 3][2 * (stp & 7)] = e0;
-              Sc[stp >> 3][2 * (stp & 7) + 1] = e1;
             }
             if ((stp & 7) == 7) {
               // the block's exponentials are all issued: its registers take the finished scores
@@ -752,7 +773,7 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
               Sn[stp >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], QA[stp & 7], Sn[stp >> 3], 0, 0, 0);
               exp_pair(stp);
             }
-            if (stp + PF < NS) rdk(kf[stp % PF], stp + PF);
+            if (stp + PF < NS) rdkp(kf[stp % PF], stp + PF, par_tag);
             if ((stp & 1) == 1 && ((stp & 7) >> 1) < kDmaGroups) {
               if (stp < 8) issue_v1(t + 1, PAR ^ 1, (stp & 7) >> 1, steady_tag);
               else if (k_on) issue_k1(t + 2, PAR, (stp & 7) >> 1, steady_tag);
@@ -773,29 +794,39 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
         // ---- PV of tile t ----
         {
           s16x4 lo[2], hi[2];
-          rdv(lo[0], 0, 0); rdv(hi[0], 0, 1);
-          rdv(lo[1], 1, 0); rdv(hi[1], 1, 1);
+          float mnext = 0.f;
+          rdv(lo[0], 0, 0, par_tag); rdv(hi[0], 0, 1, par_tag);
+          rdv(lo[1], 1, 0, par_tag); rdv(hi[1], 1, 1, par_tag);
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int stp = 0; stp < NS; ++stp) {
             const int db = stp & 3, kj = stp >> 2;
-            if (stp + 1 < NS) lds_wait2<2>(lo[stp & 1], hi[stp & 1]);
-            else lds_wait2<0>(lo[stp & 1], hi[stp & 1]);
+            // (the running maximum below passes through the wait statement, which pins one of its
+            // instructions to every MFMA)
+            if (stp + 1 < NS) lds_wait2_pin<2>(lo[stp & 1], hi[stp & 1], mnext);
+            else lds_wait2_pin<0>(lo[stp & 1], hi[stp & 1], mnext);
             const s16x4 a = lo[stp & 1], b2 = hi[stp & 1];
             const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
             OA[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), P[kj >> 1][kj & 1], OA[db], 0, 0, 0);
-            if (stp + 2 < NS) { rdv(lo[stp & 1], stp + 2, 0); rdv(hi[stp & 1], stp + 2, 1); }
+            if (stp + 2 < NS) { rdv(lo[stp & 1], stp + 2, 0, par_tag); rdv(hi[stp & 1], stp + 2, 1, par_tag); }
+            // unmasked row maximum of the scores of tile t + 1 (Sc holds them since the QK steps);
+            // without a next tile the value is not used
+            mnext = stp == 0 ? fmaxf(Sc[0][0], Sc[0][1])
+                             : fmaxf(fmaxf(mnext, Sc[stp >> 3][2 * (stp & 7)]), Sc[stp >> 3][2 * (stp & 7) + 1]);
             __builtin_amdgcn_sched_barrier(0);
           }
+          mx_carry = half_swap_max(mnext) * c;
         }
-        // the next tile reads the other buffers
+        if constexpr (PARC < 0) {
+          // the next tile reads the other buffers
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) ka[ks] -= flip;
+          for (int ks = 0; ks < 8; ++ks) ka[ks] -= flip;
 #pragma unroll
-        for (int r = 0; r < 2; ++r)
+          for (int r = 0; r < 2; ++r)
 #pragma unroll
-          for (int db = 0; db < 4; ++db) va[r][db] += flip;
-        flip = -flip;
+            for (int db = 0; db < 4; ++db) va[r][db] += flip;
+          flip = -flip;
+        }
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): K(t+2), V(t+1) and the slots have landed
         __syncthreads();
       };
@@ -832,6 +863,14 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+      {
+        float m0 = fmaxf(SX[0][0], SX[0][1]);
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int i = (b == 0 ? 2 : 0); i < 16; i += 2) m0 = fmaxf(fmaxf(m0, SX[b][i]), SX[b][i + 1]);
+        mx_carry = half_swap_max(m0) * c;
+      }
       // from here on ka reads K(t+1) in buffer 1 and va reads V(t) in buffer 0
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) ka[ks] += kBufBytes;
@@ -851,12 +890,32 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
         if (p.mask_mode == PDLLM_MASK_DENSE) open_tiles = 0;
         const int new_end = T1 - 1 < Tc + open_tiles ? T1 - 1 : Tc + open_tiles;
         int t = T0;
+        using AnyPar = std::integral_constant<int, -1>;
+        using Even = std::integral_constant<int, 0>;
+        using Odd = std::integral_constant<int, 1>;
         if constexpr (BUF) {  // (the wide-address form keeps the one general loop: it has no registers to spare)
-          for (; t < ctx_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 1>{});
-          for (; t < T1 && t < Tc; ++t) iter(t, (t - T0) & 1, SX, Generic{});
-          for (; t < new_end; ++t) iter(t, (t - T0) & 1, SX, std::integral_constant<int, 2>{});
+          // Each steady form runs unrolled by two from an even iteration on (t - T0 even: ka on buffer 1, va on
+          // buffer 0): the buffers are then immediate offsets from ka moved to buffer 0, nothing toggles and
+          // the scores of the two tiles alternate between two register sets without moves.
+          auto pairs = [&](int end, auto steady_tag) __attribute__((always_inline)) {
+            if (((t - T0) & 1) && t < end) { iter(t, 1, SX, steady_tag, AnyPar{}); ++t; }
+            if (t + 1 < end) {
+#pragma unroll
+              for (int ks = 0; ks < 8; ++ks) ka[ks] -= kBufBytes;
+              for (; t + 1 < end; t += 2) {
+                iter(t, 0, SX, steady_tag, Even{});
+                iter(t + 1, 1, SX, steady_tag, Odd{});
+              }
+#pragma unroll
+              for (int ks = 0; ks < 8; ++ks) ka[ks] += kBufBytes;
+            }
+            for (; t < end; ++t) iter(t, (t - T0) & 1, SX, steady_tag, AnyPar{});
+          };
+          pairs(ctx_end, std::integral_constant<int, 1>{});
+          for (; t < T1 && t < Tc; ++t) iter(t, (t - T0) & 1, SX, Generic{}, AnyPar{});
+          pairs(new_end, std::integral_constant<int, 2>{});
         }
-        for (; t < T1; ++t) iter(t, (t - T0) & 1, SX, Generic{});
+        for (; t < T1; ++t) iter(t, (t - T0) & 1, SX, Generic{}, AnyPar{});
       }
       // leave ka / va pointing at buffer 0 for the next piece
       if (flip > 0) {
