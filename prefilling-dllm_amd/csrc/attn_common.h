@@ -190,4 +190,106 @@ __device__ __forceinline__ void lds_wait2_pin(T& x, T& y, float& a) {
   asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(x), "+v"(y), "+v"(a) : "n"(N) : "memory");
 }
 
+// One QK step of the software-pipelined loop as a single statement, so that its order is fixed and no wait state is
+// spent between the parts: wait for the K fragment, the MFMA of the next tile's scores, the exponentials of this
+// step's two scores (their arguments t0, t1 were formed a step earlier), the arguments u0, u1 of the next step's
+// pair, then the pack of the two probabilities into one word and its contribution to the row sum.  Two vector
+// instructions lie between an exponential and the instruction that reads it (a transcendental result needs one).
+// KIND 0: first MFMA of a key block (starts from zero), 1: accumulates in place, 2 and 3: last MFMA of the block: it
+// writes `dst` (the registers of the scores this block has used up; every argument taken from them was formed
+// before this step) from the accumulator `acc`.  `keep` names the fragment the MFMA of the step before still reads.
+template <int N, int KIND>
+__device__ __forceinline__ void qk_step(f32x16& acc, f32x16& dst, const bf16x8& kf, const bf16x8& q, float& t0, float& t1,
+                                        float s2, float s3, float c, float negm, float& u0, float& u1, unsigned& pw,
+                                        float& psum, const bf16x8& keep) {
+  if constexpr (KIND == 0) {
+    asm volatile(
+        "s_waitcnt lgkmcnt(%[n])\n"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[kf], %[q], 0\n"
+        "v_exp_f32 %[t0], %[t0]\n"
+        "v_exp_f32 %[t1], %[t1]\n"
+        "v_fma_f32 %[u0], %[s2], %[c], %[nm]\n"
+        "v_fma_f32 %[u1], %[s3], %[c], %[nm]\n"
+        "v_cvt_pk_bf16_f32 %[pw], %[t0], %[t1]\n"
+        "v_dot2c_f32_bf16 %[ps], 0x3f803f80, %[pw]\n"
+        : [acc] "=&v"(acc), [t0] "+v"(t0), [t1] "+v"(t1), [u0] "=&v"(u0), [u1] "=&v"(u1), [pw] "=&v"(pw), [ps] "+v"(psum)
+        : [kf] "v"(kf), [q] "v"(q), [s2] "v"(s2), [s3] "v"(s3), [c] "s"(c), [nm] "v"(negm), [n] "n"(N), "v"(keep)
+        : "memory");
+  } else if constexpr (KIND == 1) {
+    asm volatile(
+        "s_waitcnt lgkmcnt(%[n])\n"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[kf], %[q], %[acc]\n"
+        "v_exp_f32 %[t0], %[t0]\n"
+        "v_exp_f32 %[t1], %[t1]\n"
+        "v_fma_f32 %[u0], %[s2], %[c], %[nm]\n"
+        "v_fma_f32 %[u1], %[s3], %[c], %[nm]\n"
+        "v_cvt_pk_bf16_f32 %[pw], %[t0], %[t1]\n"
+        "v_dot2c_f32_bf16 %[ps], 0x3f803f80, %[pw]\n"
+        : [acc] "+v"(acc), [t0] "+v"(t0), [t1] "+v"(t1), [u0] "=&v"(u0), [u1] "=&v"(u1), [pw] "=&v"(pw), [ps] "+v"(psum)
+        : [kf] "v"(kf), [q] "v"(q), [s2] "v"(s2), [s3] "v"(s3), [c] "s"(c), [nm] "v"(negm), [n] "n"(N), "v"(keep)
+        : "memory");
+  } else if constexpr (KIND == 3) {  // the last step of a tile: no next pair; the MFMA separates the exponentials from the pack
+    asm volatile(
+        "s_waitcnt lgkmcnt(%[n])\n"
+        "v_exp_f32 %[t0], %[t0]\n"
+        "v_exp_f32 %[t1], %[t1]\n"
+        "v_mfma_f32_32x32x16_bf16 %[dst], %[kf], %[q], %[acc]\n"
+        "v_cvt_pk_bf16_f32 %[pw], %[t0], %[t1]\n"
+        "v_dot2c_f32_bf16 %[ps], 0x3f803f80, %[pw]\n"
+        : [dst] "=&v"(dst), [t0] "+v"(t0), [t1] "+v"(t1), [pw] "=&v"(pw), [ps] "+v"(psum)
+        : [acc] "v"(acc), [kf] "v"(kf), [q] "v"(q), [n] "n"(N), "v"(keep)
+        : "memory");
+  } else {
+    asm volatile(
+        "s_waitcnt lgkmcnt(%[n])\n"
+        "v_mfma_f32_32x32x16_bf16 %[dst], %[kf], %[q], %[acc]\n"
+        "v_exp_f32 %[t0], %[t0]\n"
+        "v_exp_f32 %[t1], %[t1]\n"
+        "v_fma_f32 %[u0], %[s2], %[c], %[nm]\n"
+        "v_fma_f32 %[u1], %[s3], %[c], %[nm]\n"
+        "v_cvt_pk_bf16_f32 %[pw], %[t0], %[t1]\n"
+        "v_dot2c_f32_bf16 %[ps], 0x3f803f80, %[pw]\n"
+        : [dst] "=&v"(dst), [t0] "+v"(t0), [t1] "+v"(t1), [u0] "=&v"(u0), [u1] "=&v"(u1), [pw] "=&v"(pw), [ps] "+v"(psum)
+        : [acc] "v"(acc), [kf] "v"(kf), [q] "v"(q), [s2] "v"(s2), [s3] "v"(s3), [c] "s"(c), [nm] "v"(negm), [n] "n"(N), "v"(keep)
+        : "memory");
+  }
+}
+
+// One PV step as a single statement: wait for the V^T fragment of this step, its MFMA, and the reads of the
+// fragment two steps ahead into the registers the MFMA has just taken its operand from.  The two 64-bit transposing
+// reads of a fragment have to land in the two halves of one 128-bit operand; an asm operand cannot be addressed
+// by halves, so the two staging operands are pinned to fixed registers (v[248:251] and v[252:255]) and the text
+// names the halves.  WHICH selects the staging operand, N the outstanding LDS operations to wait for, OFF the
+// immediate offset of the reads (a negative OFF: no reads, the last two steps).  `pin` is only named: it orders
+// the vector instruction that produced it in front of this statement.
+template <int WHICH, int OFF>
+__device__ __forceinline__ void pv_read(bf16x8& a, unsigned x, unsigned y) {
+  if constexpr (WHICH == 0)
+    asm volatile("ds_read_b64_tr_b16 v[248:249], %1 offset:%3\n ds_read_b64_tr_b16 v[250:251], %2 offset:%3"
+                 : "={v[248:251]}"(a) : "v"(x), "v"(y), "n"(OFF) : "memory");
+  else
+    asm volatile("ds_read_b64_tr_b16 v[252:253], %1 offset:%3\n ds_read_b64_tr_b16 v[254:255], %2 offset:%3"
+                 : "={v[252:255]}"(a) : "v"(x), "v"(y), "n"(OFF) : "memory");
+}
+template <int WHICH, int N, int OFF, typename P4>
+__device__ __forceinline__ void pv_step(f32x16& o, bf16x8& a, const P4& p, unsigned x, unsigned y, float pin) {
+  if constexpr (OFF >= 0) {
+    if constexpr (WHICH == 0)
+      asm volatile("s_waitcnt lgkmcnt(%6)\n v_mfma_f32_32x32x16_bf16 %0, v[248:251], %2, %0\n"
+                   "ds_read_b64_tr_b16 v[248:249], %3 offset:%7\n ds_read_b64_tr_b16 v[250:251], %4 offset:%7"
+                   : "+v"(o), "+{v[248:251]}"(a) : "v"(p), "v"(x), "v"(y), "v"(pin), "n"(N), "n"(OFF) : "memory");
+    else
+      asm volatile("s_waitcnt lgkmcnt(%6)\n v_mfma_f32_32x32x16_bf16 %0, v[252:255], %2, %0\n"
+                   "ds_read_b64_tr_b16 v[252:253], %3 offset:%7\n ds_read_b64_tr_b16 v[254:255], %4 offset:%7"
+                   : "+v"(o), "+{v[252:255]}"(a) : "v"(p), "v"(x), "v"(y), "v"(pin), "n"(N), "n"(OFF) : "memory");
+  } else {
+    if constexpr (WHICH == 0)
+      asm volatile("s_waitcnt lgkmcnt(%4)\n v_mfma_f32_32x32x16_bf16 %0, v[248:251], %2, %0"
+                   : "+v"(o), "+{v[248:251]}"(a) : "v"(p), "v"(pin), "n"(N) : "memory");
+    else
+      asm volatile("s_waitcnt lgkmcnt(%4)\n v_mfma_f32_32x32x16_bf16 %0, v[252:255], %2, %0"
+                   : "+v"(o), "+{v[252:255]}"(a) : "v"(p), "v"(pin), "n"(N) : "memory");
+  }
+}
+
 }  // namespace pdllm

@@ -730,49 +730,44 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
         // ---- exponentials of tile t, two per step, between the MFMAs of QK(t+1) ----
         float negM = (MA == -INFINITY) ? 0.f : -MA;
         f32x16 Sn[2];
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) Sn[b][i] = 0.f;
-        bf16x8 P[2][2];
+        typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+        u32x4 PW[2][2];  // probabilities of tile t, two bf16 per word: the B operands of PV
         const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
         float psum = 0.f;
-        auto exp_pair = [&](int stp) __attribute__((always_inline)) {
-          const int b = stp >> 3, i = 2 * (stp & 7);
-          const bf16x2 pr = {(__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(Sc[b][i], c, negM)),
-                             (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(Sc[b][i + 1], c, negM))};
-          psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);
-          P[b][i >> 3][i & 7] = pr[0];
-          P[b][i >> 3][(i & 7) + 1] = pr[1];
-        };
         if (has_next) {
           bf16x8 kf[PF];
 #pragma unroll
           for (int i = 0; i < PF; ++i) rdkp(kf[i], i, par_tag);
           bf16x8 used = kf[0];  // fragment of the MFMA issued in the step before
+          // arguments of the first pair of exponentials; every step forms those of the next one
+          float t0 = __builtin_fmaf(Sc[0][0], c, negM), t1 = __builtin_fmaf(Sc[0][1], c, negM);
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int stp = 0; stp < NS; ++stp) {
-            {
-              // wait for this step's K fragment; the subtrahend of the step's exponentials and the running
-              // sum of the step before pass through the same statement: the step's arithmetic stays behind
-              // the wait, the arithmetic of the step before in front of it.  (The scores themselves do not
-              // pass through it: a tied operand that is one element of a 16-register tuple costs a move.)
-              const int young = NS - 1 - stp < PF - 1 ? NS - 1 - stp : PF - 1;
-              if (young == 3) lds_wait_pin<3>(kf[stp % PF], negM, psum, used);
-              else if (young == 2) lds_wait_pin<2>(kf[stp % PF], negM, psum, used);
-              else if (young == 1) lds_wait_pin<1>(kf[stp % PF], negM, psum, used);
-              else lds_wait_pin<0>(kf[stp % PF], negM, psum, used);
-              used = kf[stp % PF];
-            }
-            if ((stp & 7) == 7) {
-              // the block's exponentials are all issued: its registers take the finished scores
-              exp_pair(stp);
-              Sc[stp >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], QA[7], Sn[stp >> 3], 0, 0, 0);
-            } else {
-              Sn[stp >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[stp % PF], QA[stp & 7], Sn[stp >> 3], 0, 0, 0);
-              exp_pair(stp);
-            }
+            const int b = stp >> 3;
+            const int nb = (stp + 1) >> 3, ni = 2 * ((stp + 1) & 7);  // the next step's pair of scores
+            const float s2 = stp + 1 < NS ? Sc[nb & 1][ni] : 0.f, s3 = stp + 1 < NS ? Sc[nb & 1][ni + 1] : 0.f;
+            float u0 = 0.f, u1 = 0.f;
+            unsigned pw;
+            constexpr int kLast = NS - 1;
+            const int young = NS - 1 - stp < PF - 1 ? NS - 1 - stp : PF - 1;
+            // (one statement per step: wait for the K fragment, MFMA, exponentials, next arguments, pack, row sum;
+            // the last MFMA of a key block writes into the registers of the scores the block has used up)
+#define PDLLM_QK_STEP(KIND, ACC, DST)                                                                                 \
+  do {                                                                                                                \
+    if (young == 2) qk_step<2, KIND>(ACC, DST, kf[stp % PF], QA[stp & 7], t0, t1, s2, s3, c, negM, u0, u1, pw, psum, used);      \
+    else if (young == 1) qk_step<1, KIND>(ACC, DST, kf[stp % PF], QA[stp & 7], t0, t1, s2, s3, c, negM, u0, u1, pw, psum, used); \
+    else qk_step<0, KIND>(ACC, DST, kf[stp % PF], QA[stp & 7], t0, t1, s2, s3, c, negM, u0, u1, pw, psum, used);                 \
+  } while (0)
+            if (stp == kLast) PDLLM_QK_STEP(3, Sn[b], Sc[b]);
+            else if ((stp & 7) == 7) PDLLM_QK_STEP(2, Sn[b], Sc[b]);
+            else if ((stp & 7) == 0) PDLLM_QK_STEP(0, Sn[b], Sn[b]);
+            else PDLLM_QK_STEP(1, Sn[b], Sn[b]);
+#undef PDLLM_QK_STEP
+            used = kf[stp % PF];
+            PW[b][(stp & 7) >> 2][stp & 3] = pw;
+            t0 = u0;
+            t1 = u1;
             if (stp + PF < NS) rdkp(kf[stp % PF], stp + PF, par_tag);
             if ((stp & 1) == 1 && ((stp & 7) >> 1) < kDmaGroups) {
               if (stp < 8) issue_v1(t + 1, PAR ^ 1, (stp & 7) >> 1, steady_tag);
@@ -787,34 +782,45 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
           else if (t + 3 < T1) load_slots(t + 3);
         } else {
 #pragma unroll
-          for (int stp = 0; stp < NS; ++stp) exp_pair(stp);
+          for (int stp = 0; stp < NS; ++stp) {
+            const int b = stp >> 3, i = 2 * (stp & 7);
+            const bf16x2 pr = {(__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(Sc[b][i], c, negM)),
+                               (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(Sc[b][i + 1], c, negM))};
+            psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);
+            PW[b][(stp & 7) >> 2][stp & 3] = __builtin_bit_cast(unsigned, pr);
+          }
         }
         lA += psum;
         __builtin_amdgcn_sched_barrier(0);
         // ---- PV of tile t ----
         {
-          s16x4 lo[2], hi[2];
+          // V^T fragments of step stp in staging operand stp & 1 (attn_common.h: pv_step); the offset of a
+          // fragment inside the tile: key block kj = stp >> 2 (16 keys each), buffer by the parity tag
+          constexpr int vbase = kTileBytes + (PARC == 1 ? kBufBytes : 0);
+          bf16x8 stg0, stg1;
           float mnext = 0.f;
-          rdv(lo[0], 0, 0, par_tag); rdv(hi[0], 0, 1, par_tag);
-          rdv(lo[1], 1, 0, par_tag); rdv(hi[1], 1, 1, par_tag);
+          pv_read<0, vbase>(stg0, va[0][0], va[1][0]);
+          pv_read<1, vbase>(stg1, va[0][1], va[1][1]);
           __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int stp = 0; stp < NS; ++stp) {
-            const int db = stp & 3, kj = stp >> 2;
-            // (the running maximum below passes through the wait statement, which pins one of its
-            // instructions to every MFMA)
-            if (stp + 1 < NS) lds_wait2_pin<2>(lo[stp & 1], hi[stp & 1], mnext);
-            else lds_wait2_pin<0>(lo[stp & 1], hi[stp & 1], mnext);
-            const s16x4 a = lo[stp & 1], b2 = hi[stp & 1];
-            const s16x8 both = {a[0], a[1], a[2], a[3], b2[0], b2[1], b2[2], b2[3]};
-            OA[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), P[kj >> 1][kj & 1], OA[db], 0, 0, 0);
-            if (stp + 2 < NS) { rdv(lo[stp & 1], stp + 2, 0, par_tag); rdv(hi[stp & 1], stp + 2, 1, par_tag); }
-            // unmasked row maximum of the scores of tile t + 1 (Sc holds them since the QK steps);
-            // without a next tile the value is not used
-            mnext = stp == 0 ? fmaxf(Sc[0][0], Sc[0][1])
-                             : fmaxf(fmaxf(mnext, Sc[stp >> 3][2 * (stp & 7)]), Sc[stp >> 3][2 * (stp & 7) + 1]);
-            __builtin_amdgcn_sched_barrier(0);
-          }
+#define PDLLM_PV_STEP(STP)                                                                                             \
+  do {                                                                                                                 \
+    constexpr int stp = STP, db = stp & 3, kj = stp >> 2, nx = stp + 2;                                                 \
+    constexpr int off = nx < NS ? vbase + (nx >> 2) * 16 * kRowBytes : -1;                                              \
+    if constexpr ((stp & 1) == 0)                                                                                       \
+      pv_step<0, (stp + 1 < NS ? 2 : 0), off>(OA[db], stg0, PW[kj >> 1][kj & 1], va[0][nx & 3], va[1][nx & 3], mnext);  \
+    else                                                                                                                \
+      pv_step<1, (stp + 1 < NS ? 2 : 0), off>(OA[db], stg1, PW[kj >> 1][kj & 1], va[0][nx & 3], va[1][nx & 3], mnext);  \
+    /* unmasked row maximum of the scores of tile t + 1 (Sc holds them since the QK steps), one instruction      */  \
+    /* between two steps; without a next tile the value is not used                                              */  \
+    mnext = stp == 0 ? fmaxf(Sc[0][0], Sc[0][1])                                                                        \
+                     : fmaxf(fmaxf(mnext, Sc[stp >> 3][2 * (stp & 7)]), Sc[stp >> 3][2 * (stp & 7) + 1]);               \
+    __builtin_amdgcn_sched_barrier(0);                                                                                  \
+  } while (0)
+          PDLLM_PV_STEP(0); PDLLM_PV_STEP(1); PDLLM_PV_STEP(2); PDLLM_PV_STEP(3);
+          PDLLM_PV_STEP(4); PDLLM_PV_STEP(5); PDLLM_PV_STEP(6); PDLLM_PV_STEP(7);
+          PDLLM_PV_STEP(8); PDLLM_PV_STEP(9); PDLLM_PV_STEP(10); PDLLM_PV_STEP(11);
+          PDLLM_PV_STEP(12); PDLLM_PV_STEP(13); PDLLM_PV_STEP(14); PDLLM_PV_STEP(15);
+#undef PDLLM_PV_STEP
           mx_carry = half_swap_max(mnext) * c;
         }
         if constexpr (PARC < 0) {
