@@ -1350,7 +1350,7 @@ static int compute_units() {
   return cached[dev];
 }
 
-static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
+static AttnPlan compute_plan(const pdllm_attn_desc* d, bool prefill) {
   const int G = d->num_q_heads / d->num_kv_heads;
   const long rows = (long)d->max_q_len * G;
   const long nblk = (rows + 31) / 32;
@@ -1361,7 +1361,7 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
   const int cus = compute_units();
   // kPiece: what a piece costs outside its tile loop (three round trips to memory before the first MFMA, the
   // last PV, the partial rows): about 3.2 tiles of a 4-wave workgroup
-  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 4.3, kWide = 1.25;
+  constexpr double kFixed = 0.35, kPair = 0.65, kPiece = 4.3, kWide = 1.45;
   constexpr int kStaticLds = 66 * 1024;
   static const int js[] = {1, 2, 4, 5, 6, 8};
   static const double upw[] = {0.45, 0.75, 1.0, 1.25, 1.5, 1.0};
@@ -1489,6 +1489,35 @@ static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
     best = {4, (int)row_tiles, (int)T, (int)T, (int)(units * row_tiles * T), 1, (int)(units * row_tiles), 0, 0};
   }
   return best;
+}
+
+// The plan depends on a handful of descriptor fields; every launch asks for it, and laying out the candidates costs
+// several microseconds of host time -- as much as a small launch runs on the GPU.  Each host thread remembers the last
+// few plans it computed.
+static AttnPlan make_plan(const pdllm_attn_desc* d, bool prefill) {
+  struct Key {
+    int64_t n_req;
+    int32_t hq, hkv, q_len, ctx, kv_dtype, mask_mode, rows, splits, tiles, cus;
+    bool prefill, has_cache;
+    bool operator==(const Key& o) const {
+      return n_req == o.n_req && hq == o.hq && hkv == o.hkv && q_len == o.q_len && ctx == o.ctx && kv_dtype == o.kv_dtype &&
+             mask_mode == o.mask_mode && rows == o.rows && splits == o.splits && tiles == o.tiles && cus == o.cus &&
+             prefill == o.prefill && has_cache == o.has_cache;
+    }
+  };
+  struct Entry { Key key; AttnPlan plan; bool used; };
+  static thread_local Entry cache[8] = {};
+  static thread_local int next = 0;
+  const Key key = {d->n_req, d->num_q_heads, d->num_kv_heads, d->max_q_len, d->max_ctx_len, d->kv_dtype, d->mask_mode,
+                   d->rows_per_group, d->num_splits, d->tiles_per_workgroup, compute_units(), prefill, d->k_cache != nullptr};
+  for (const Entry& e : cache)
+    if (e.used && e.key == key) return e.plan;
+  Entry& e = cache[next];
+  next = (next + 1) & 7;
+  e.key = key;
+  e.plan = compute_plan(d, prefill);
+  e.used = true;
+  return e.plan;
 }
 
 static bool needs_own_table(const pdllm_attn_desc* d, bool prefill) {

@@ -143,8 +143,13 @@ def test_planner_lays_out_the_set_cut_without_a_gpu():
     loads = [(min(a + span, rt * tail) - a, (min(a + span, rt * tail) - 1) // tail - a // tail + 1)
              for a in range(0, rt * tail, span)]
     assert len(loads) == k - rt and max(p for _, p in loads) == 2 and sum(p for _, p in loads) == 13
-    # 32 response rows only: the eight-wave kernel, every (request, KV head) cut into eight aligned pieces
+    # 32 response rows only: the 224 rows of a (request, KV head) are two row groups, each cut into eight aligned
+    # pieces (two workgroups per CU); the eight-wave kernel on request
     f, kernel = _plan_text(_decode_desc(8, 32, 4096))
+    assert kernel == "attn_fwd_kernel" and (f["row_blocks"], f["grid"], f["span"], f["head"], f["pieces"]) == ("4", "512", "9", "0", "8")
+    d = _decode_desc(8, 32, 4096)
+    d.rows_per_group = 256
+    f, kernel = _plan_text(d)
     assert kernel == "attn_fwd2_kernel" and (f["row_blocks"], f["grid"], f["span"], f["head"]) == ("8", "256", "9", "0")
     # fp8 pages, 160 rows per head: one group of five row blocks, two aligned pieces
     f, kernel = _plan_text(_decode_desc(4, 160, 16 * 1025, hq=32, hkv=32, fp8=True))
