@@ -159,6 +159,31 @@ def test_planner_lays_out_the_set_cut_without_a_gpu():
     assert f["pieces"] == "1" and f["partial_row_bytes"] == "0"
 
 
+def test_remembered_plans_equal_fresh_ones():
+    """The library remembers the last eight plans per host thread.  More shapes than that, visited twice in an order
+    that evicts every entry in between, and from a second thread: every answer equals the first one."""
+    import threading
+    shapes = [(n, q, c, hq, hkv, fp8) for n in (1, 3, 8) for q in (32, 160) for c in (1024, 4096)
+              for hq, hkv, fp8 in ((28, 4, False), (32, 32, True))]
+    assert len(shapes) > 8
+    first = [_plan_text(_decode_desc(n, q, c, hq=hq, hkv=hkv, fp8=fp8)) for n, q, c, hq, hkv, fp8 in shapes]
+    assert len({str(x) for x in first}) > 8          # the shapes really have different plans
+    again = [_plan_text(_decode_desc(n, q, c, hq=hq, hkv=hkv, fp8=fp8)) for n, q, c, hq, hkv, fp8 in shapes]
+    assert again == first
+    for n, q, c, hq, hkv, fp8 in shapes[:3]:         # the same shape back to back: served from the memory
+        d = _decode_desc(n, q, c, hq=hq, hkv=hkv, fp8=fp8)
+        assert _plan_text(d) == _plan_text(d)
+        d.rows_per_group = 128                       # a forced field is part of the key
+        forced = _plan_text(d)
+        d.rows_per_group = 0
+        assert _plan_text(d) == first[shapes.index((n, q, c, hq, hkv, fp8))] and forced[0]["row_blocks"] == "4"
+    other = []
+    t = threading.Thread(target=lambda: other.extend(
+        _plan_text(_decode_desc(n, q, c, hq=hq, hkv=hkv, fp8=fp8)) for n, q, c, hq, hkv, fp8 in shapes))
+    t.start(); t.join()
+    assert other == first
+
+
 def test_page_pool_semantics():
     """What callers of the reference's allocator observe (fastdllm_engine.py:88-167): pages are handed out in the
     order they became free, refcounts, the exhaustion error, hash-keyed prefix reuse and eviction."""
