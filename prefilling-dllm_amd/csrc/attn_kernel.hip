@@ -573,7 +573,10 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
   // elements of tile t.  K therefore runs one tile ahead of V in the buffers: iteration t
   // reads K(t+1) and V(t) and copies K(t+2) and V(t+1).  The last MFMA of a key block writes
   // into the registers the finished exponentials have just released, so the new scores are in
-  // place for the next iteration without moves.
+  // place for the next iteration without moves.  Every QK step and every PV step is one asm
+  // statement (attn_common.h: qk_step, pv_step): its order is fixed, the MFMA comes first and
+  // nothing is inserted between its parts.  Between the PV steps runs the row maximum of tile
+  // t + 1, so that an iteration over an unmasked tile starts with its maximum known.
   // ------------------------------------------------------------------------------------------
   constexpr bool PIPELINED = (J == 4 || J == 8) && !KV_FP8;
   if constexpr (PIPELINED) {
