@@ -15,6 +15,8 @@ attention is computed for every row and read at the anchors."""
 from __future__ import annotations
 
 import os
+from dataclasses import dataclass
+from typing import Optional
 
 import torch
 from torch import nn
@@ -51,8 +53,12 @@ class Attention(nn.Module):
         # A decode step over a cached prefix stores its active rows inside the attention call (their slots lie
         # behind the context the same call reads, ENG:497); every other case stores first, as the reference does.
         max_ctx = 0 if context.is_prefill else int(context.max_context_len) or max(int(context.max_seqlen_k) - 1, 0)
+        # (precondition: no active slot lies inside a visible prefix range; `context.store_before_attention`
+        # restores the reference's order for callers that break it, PDLLM_DEBUG_CHECKS=1 verifies it on the host)
         store_in_call = (has_cache and context.need_kv_cache_store and not context.is_prefill and max_ctx > 0
-                         and context.slot_mapping is not None)
+                         and context.slot_mapping is not None and not context.store_before_attention)
+        if store_in_call and os.environ.get("PDLLM_DEBUG_CHECKS", "0") == "1":
+            self._check_store_after_attention(context, k_cache.shape[1])
         if has_cache and context.need_kv_cache_store and not store_in_call:
             ops.store_kvcache_unified_layout(k, v, k_cache, v_cache, context.slot_mapping, self.model_type, context)
 
@@ -63,7 +69,12 @@ class Attention(nn.Module):
                 raise ValueError(f"block_mask must be [rows, keys] with one row per active token, got {tuple(dense.shape)}")
             if dense.shape[1] != q.shape[0]:
                 # the reference's decode form [Nq, sum(ctx + Sq)] (utils/context.py:85-98): keep the active columns
-                dense = self._active_columns(dense, context)
+                # (reduced once per context, not once per layer: every layer of a step passes the same mask)
+                held = getattr(context, "_active_mask_of", None)
+                if held is None or held[0] is not dense:
+                    held = (dense, self._active_columns(dense, context))
+                    context._active_mask_of = held
+                dense = held[1]
                 if dense is None:          # nothing hidden: the bidirectional block needs no mask tensor
                     mask_mode = "full"
         if context.is_prefill:
@@ -88,14 +99,43 @@ class Attention(nn.Module):
         return o.view(-1, self.num_heads * self.head_dim)
 
     @staticmethod
+    def _check_store_after_attention(context: ContextForDiffusionLM, page_size: int) -> None:
+        """Debug check of the in-call store's precondition: no slot that receives an active row is the slot of a
+        visible prefix key of the same call (host-side, synchronises)."""
+        slots = context.slot_mapping[context.slot_mapping >= 0].long()
+        if slots.numel() == 0 or context.block_tables is None:
+            return
+        if context.ranges is not None:
+            ptr, start, length = (t.tolist() for t in context.ranges[:3])
+            spans = [[(start[i], length[i]) for i in range(ptr[r], ptr[r + 1])] for r in range(len(ptr) - 1)]
+        else:
+            spans = [[(0, int(n))] for n in context.context_lens.tolist()]
+        for r, req_spans in enumerate(spans):
+            table = context.block_tables[r].long()
+            for first, n in req_spans:
+                if n <= 0:
+                    continue
+                tok = torch.arange(first, first + n, device=slots.device)
+                visible = table[tok // page_size] * page_size + tok % page_size
+                if torch.isin(visible, slots).any().item():
+                    raise RuntimeError("an active row's slot lies inside a visible prefix range: set "
+                                       "context.store_before_attention to store in front of the attention")
+
+    @staticmethod
     def _active_columns(mask: torch.Tensor, context: ContextForDiffusionLM):
         """[Nq, sum(ctx_s + Sq_s)] block-diagonal decode mask of the reference -> [Nq, Nq] over the active keys
         (None when no active key is hidden)."""
         from .context import active_block_mask
         if context.is_prefill or context.context_lens is None or context.cu_seqlens_q is None:
             raise ValueError(f"block_mask of shape {tuple(mask.shape)} does not match {mask.shape[0]} active rows")
+        # (the context's host-side lengths when it carries them: no transfer)
+        if context.seq_lens is not None and len(context.seq_lens) == context.context_lens.numel():
+            cu = [0]
+            for n in context.seq_lens:
+                cu.append(cu[-1] + int(n))
+        else:
+            cu = [int(x) for x in context.cu_seqlens_q.tolist()]
         ctx = [int(x) for x in context.context_lens.tolist()]
-        cu = [int(x) for x in context.cu_seqlens_q.tolist()]
         if mask.shape[1] != sum(ctx) + cu[-1]:
             raise ValueError(f"block_mask has {mask.shape[1]} key columns, expected {cu[-1]} (active) or "
                              f"{sum(ctx) + cu[-1]} (contexts + active)")
@@ -117,21 +157,26 @@ class Attention(nn.Module):
 
     def _paged_prompt(self, state, full_k, full_v, extra: int):
         """The layer's full prompt K/V [S, Hkv, d] as pages of a cache of its own (where the reference concatenates,
-        attention_v4.py:120-125) with room for `extra` more tokens.  The copy is kept in the state between steps and
-        made again when the prompt tensors change."""
+        attention_v4.py:120-125) with room for `extra` more tokens.  The copy lives in the state between steps and
+        is tied to the prompt tensor *objects* it was made from (the entry holds them, so their storage cannot be
+        freed and handed to another tensor while the copy is in use); a caller that rewrites those tensors in place
+        drops the copy with `state.pop("_paged_prompt", None)` or bumps `state["prompt_generation"]`.  The copy
+        doubles the prompt K/V of the layer in device memory for as long as the state lives."""
         page, n_prompt = 256, int(full_k.shape[0])
         pages = (n_prompt + extra + page - 1) // page
-        key = (full_k.data_ptr(), full_v.data_ptr(), n_prompt, full_k._version, full_v._version)
+        generation = state.get("prompt_generation", 0)
         held = state.setdefault("_paged_prompt", {})
         ent = held.get(self.layer_idx)
-        if ent is None or ent[0] != key or ent[1].shape[0] < pages:
+        fresh = (ent is not None and ent["k"] is full_k and ent["v"] is full_v and ent["n"] == n_prompt
+                 and ent["generation"] == generation and ent["kc"].shape[0] >= pages)
+        if not fresh:
             kc = torch.empty((pages, page, self.num_kv_heads, self.head_dim), dtype=full_k.dtype, device=full_k.device)
             vc = torch.empty_like(kc)
             kc.view(-1, self.num_kv_heads, self.head_dim)[:n_prompt].copy_(full_k)
             vc.view(-1, self.num_kv_heads, self.head_dim)[:n_prompt].copy_(full_v)
-            ent = (key, kc, vc)
+            ent = {"k": full_k, "v": full_v, "n": n_prompt, "generation": generation, "kc": kc, "vc": vc}
             held[self.layer_idx] = ent
-        return ent[1], ent[2]
+        return ent["kc"], ent["vc"]
 
     def _maybe_apply_decode_delta(self, o, q, k_new, v_new, context, mask_mode="full", active_mask=None):
         """attention_v4.py:86-166.  The packed active rows are one sequence, as in the reference; active_mask is the
@@ -189,93 +234,122 @@ class Attention(nn.Module):
 
     def _maybe_prefill_sparse_attention(self, q, k, v, context):
         """attention_v4.py:168-293.  None = not active, the caller runs the ordinary prefill."""
+        if self.model_type != "diffusion_lm":
+            return None
         state = getattr(context, "prefill_sparse_state", None)
-        if not state or not state.get("enabled", False):
+        plan = _SparsePrefill.parse(state, self.layer_idx, q.shape[0], self.num_heads, context.block_mask, q.device,
+                                    q.dtype)
+        if plan is None:
             return None
-        if self.model_type != "diffusion_lm" or self.layer_idx < 0:
-            return None
-        keep_by_layer = state.get("keep_indices")
-        if keep_by_layer is None or self.layer_idx >= len(keep_by_layer):
-            return None
-        base_mask = context.block_mask
-        if base_mask is None:
-            return None
-        seq_len, dev = q.shape[0], q.device
-        layer_keep = keep_by_layer[self.layer_idx]
-        if layer_keep is None or layer_keep.numel() == 0:
-            return None
-        valid_keep = layer_keep.to(device=dev, dtype=torch.long).reshape(-1)
-        valid_keep = valid_keep[(valid_keep >= 0) & (valid_keep < seq_len)]
-        if valid_keep.numel() == 0:
-            return None
-        key_mask = torch.zeros(seq_len, dtype=torch.bool, device=dev)
-        key_mask[valid_keep] = True
-        full_prompt_len = int(state.get("full_prompt_len", seq_len))
-        if 0 <= full_prompt_len < seq_len:
-            key_mask[full_prompt_len:] = True
-        if state.get("debug", False):
-            active_keys = int(key_mask.sum().item())
-            state["union_min"] = min(int(state.get("union_min", active_keys)), active_keys)
-            state["union_max"] = max(int(state.get("union_max", active_keys)), active_keys)
-        base_mask = base_mask.to(device=dev, dtype=torch.bool)
-        one_seq = torch.tensor([0, seq_len], dtype=torch.int32, device=dev)
+        seq_len = q.shape[0]
+        one_seq = torch.tensor([0, seq_len], dtype=torch.int32, device=q.device)
 
         def attend(mask):
             return ops.sparse_decode_attention(q, k, v, None, None, None, one_seq, max_q_len=seq_len, max_ctx_len=0,
                                                mask_mode="dense", mask=mask, sm_scale=self.scale)
 
-        o_sparse = attend(base_mask & key_mask.unsqueeze(0))
-        delta_mode = (state.get("delta_mode") or "none").lower()
-        if delta_mode in {"none", "off", "0", ""}:
+        if plan.debug:
+            n_keys = int(plan.keys.sum().item())
+            state["union_min"] = min(int(state.get("union_min", n_keys)), n_keys)
+            state["union_max"] = max(int(state.get("union_max", n_keys)), n_keys)
+        o_sparse = attend(plan.rows_mask & plan.keys.unsqueeze(0))
+        if plan.anchor is None:            # no correction asked for, or no anchor row in this sequence
             return o_sparse
-        if delta_mode not in {"s4_left3", "delta_s4_left3", "sampled_delta_s4_left3"}:
-            raise ValueError(f"Unsupported prefill_delta_mode: {delta_mode}")
-        ap = ops.anchor_params(state, seq_len)
-        if ap is None:
-            return o_sparse
-        stride, offset, left, right, direction = ap
-
-        selection_mode = (state.get("selection_mode") or "none").lower()
-        selection_dense = state.get("selection_dense")
-        sel = counts = None
-        if selection_mode in {"selection_dense_replace", "selection_dense_add"} and selection_dense:
-            outputs_by_layer = selection_dense.get("outputs") if isinstance(selection_dense, dict) else None
-            counts_by_layer = selection_dense.get("counts") if isinstance(selection_dense, dict) else None
-            if outputs_by_layer is not None and self.layer_idx < len(outputs_by_layer):
-                layer_outputs = outputs_by_layer[self.layer_idx]
-                if layer_outputs is not None and layer_outputs.shape[0] > 0 and layer_outputs.shape[1] == self.num_heads:
-                    sel = layer_outputs.to(device=dev, dtype=o_sparse.dtype).contiguous()
-                    if counts_by_layer is not None and self.layer_idx < len(counts_by_layer) and \
-                            counts_by_layer[self.layer_idx] is not None:
-                        counts = counts_by_layer[self.layer_idx].to(dev)
-        scale = float(state.get("scale", 1.0))
+        stride, offset, left, right, direction = plan.anchor
         kw = dict(max_q_len=seq_len, stride=stride, anchor_offset=offset, left=left, right=right, direction=direction,
-                  scale=scale)
-        anchors = torch.arange(offset, seq_len, stride, device=dev)
+                  scale=plan.scale)
+        anchors = torch.arange(offset, seq_len, stride, device=q.device)
 
-        def any_valid():
-            in_range = anchors < sel.shape[0]
-            if counts is None:
-                return bool(in_range.any().item())
-            safe = anchors.clamp_max(sel.shape[0] - 1)
-            return bool(((counts.index_select(0, safe) > 0) & in_range).any().item())
-
-        if selection_mode == "selection_dense_replace":
-            if sel is None or not any_valid():
+        if plan.mode == "replace":
+            # the selection's rows stand in for the dense attention of the anchors; without a usable row: no correction
+            if plan.sel is None or not plan.selection_covers(anchors):
                 return o_sparse
-            out = ops.anchor_delta_add(o_sparse, None, one_seq, sel=sel, sel_counts=counts, sel_mode="replace", **kw)
+            out = ops.anchor_delta_add(o_sparse, None, one_seq, sel=plan.sel, sel_counts=plan.sel_counts,
+                                       sel_mode="replace", **kw)
             state["selection_used_calls"] = int(state.get("selection_used_calls", 0)) + 1
-            dense = None
+        elif plan.mode == "add" and plan.sel is not None:
+            out = ops.anchor_delta_add(o_sparse, attend(plan.rows_mask), one_seq, sel=plan.sel,
+                                       sel_counts=plan.sel_counts, sel_mode="add", sel_scale=plan.sel_scale, **kw)
+            state["selection_used_calls"] = int(state.get("selection_used_calls", 0)) + 1
         else:
-            dense = attend(base_mask)
-            if selection_mode == "selection_dense_add" and sel is not None:
-                out = ops.anchor_delta_add(o_sparse, dense, one_seq, sel=sel, sel_counts=counts, sel_mode="add",
-                                           sel_scale=float(state.get("selection_scale", 1.0)), **kw)
-                state["selection_used_calls"] = int(state.get("selection_used_calls", 0)) + 1
-            else:
-                out = ops.anchor_delta_add(o_sparse, dense, one_seq, **kw)
-        if state.get("debug", False):
+            out = ops.anchor_delta_add(o_sparse, attend(plan.rows_mask), one_seq, **kw)
+        if plan.debug:
             # largest |out - o_sparse| over the anchor rows stands in for the reference's max |delta|
             diff = (out.index_select(0, anchors).float() - o_sparse.index_select(0, anchors).float()).abs()
             self._debug_stats(state, float(diff.max().item()) if diff.numel() else 0.0, int(anchors.numel()))
         return out
+
+
+_DELTA_OFF = frozenset({"none", "off", "0", ""})
+_DELTA_ON = frozenset({"s4_left3", "delta_s4_left3", "sampled_delta_s4_left3"})
+_SELECTION_MODES = {"selection_dense_replace": "replace", "selection_dense_add": "add"}
+
+
+@dataclass
+class _SparsePrefill:
+    """One layer's view of the `prefill_sparse_state` dictionary (attention_v4.py:171-232), read once.
+
+    keys        [S] bool, the key columns the sparse pass may see: the layer's keep list and everything from
+                `full_prompt_len` on
+    rows_mask   [S, S] bool, the context's block mask
+    anchor      (stride, offset, left, right, direction) of the correction, None = sparse pass only
+    mode        "plain" | "replace" | "add": where the anchors' denser rows come from
+    sel         [n, Hq, d] ready-made anchor rows of this layer (selection modes), with per-row counts
+    """
+    keys: torch.Tensor
+    rows_mask: torch.Tensor
+    anchor: Optional[tuple] = None
+    mode: str = "plain"
+    sel: Optional[torch.Tensor] = None
+    sel_counts: Optional[torch.Tensor] = None
+    scale: float = 1.0
+    sel_scale: float = 1.0
+    debug: bool = False
+
+    @staticmethod
+    def _layer_entry(table, layer_idx):
+        if table is None or not 0 <= layer_idx < len(table):
+            return None
+        return table[layer_idx]
+
+    @classmethod
+    def parse(cls, state, layer_idx, seq_len, num_heads, block_mask, dev, dtype):
+        if not state or not state.get("enabled", False) or layer_idx < 0 or block_mask is None:
+            return None
+        keep = cls._layer_entry(state.get("keep_indices"), layer_idx)
+        if keep is None or keep.numel() == 0:
+            return None
+        keep = keep.to(device=dev, dtype=torch.long).flatten()
+        keep = keep[(keep >= 0) & (keep < seq_len)]
+        if keep.numel() == 0:
+            return None
+        keys = torch.zeros(seq_len, dtype=torch.bool, device=dev).index_fill_(0, keep, True)
+        prompt_end = int(state.get("full_prompt_len", seq_len))
+        if 0 <= prompt_end < seq_len:
+            keys[prompt_end:] = True
+        plan = cls(keys=keys, rows_mask=block_mask.to(device=dev, dtype=torch.bool),
+                   scale=float(state.get("scale", 1.0)), sel_scale=float(state.get("selection_scale", 1.0)),
+                   debug=bool(state.get("debug", False)))
+        delta_mode = (state.get("delta_mode") or "none").lower()
+        if delta_mode in _DELTA_OFF:
+            return plan
+        if delta_mode not in _DELTA_ON:
+            raise ValueError(f"Unsupported prefill_delta_mode: {delta_mode}")
+        plan.anchor = ops.anchor_params(state, seq_len)
+        plan.mode = _SELECTION_MODES.get((state.get("selection_mode") or "none").lower(), "plain")
+        ready = state.get("selection_dense")
+        if plan.mode != "plain" and isinstance(ready, dict):
+            rows = cls._layer_entry(ready.get("outputs"), layer_idx)
+            if rows is not None and rows.dim() == 3 and rows.shape[0] > 0 and rows.shape[1] == num_heads:
+                plan.sel = rows.to(device=dev, dtype=dtype).contiguous()
+                counts = cls._layer_entry(ready.get("counts"), layer_idx)
+                plan.sel_counts = None if counts is None else counts.to(dev)
+        return plan
+
+    def selection_covers(self, anchors) -> bool:
+        """Does the selection hold a usable row (in range, count > 0) for at least one anchor?"""
+        n = self.sel.shape[0]
+        usable = anchors < n
+        if self.sel_counts is not None:
+            usable = usable & (self.sel_counts.index_select(0, anchors.clamp_max(n - 1)) > 0)
+        return bool(usable.any().item())

@@ -39,6 +39,12 @@ class ContextForDiffusionLM:
     # first context_lens[r] tokens of each page table (the reference's decode context)
     ranges: Any = None
     max_context_len: int = 0
+    # A decode step over a cached prefix normally stores its active rows inside the attention call, after the
+    # kernel has read the cache.  That equals the reference's store-then-attend order (attention_v4.py:328-331)
+    # only while no active slot lies inside a visible prefix range -- true for the reference's own callers
+    # (fastdllm_engine.py:497: the block's slots follow the context).  A caller that rewrites visible context
+    # rows sets this flag: the store then runs as a launch of its own in front of the attention.
+    store_before_attention: bool = False
 
     def __post_init__(self):
         if self.seq_lens_ts is not None and self.context_lens is not None:
@@ -65,19 +71,26 @@ def active_block_mask(masks) -> Optional[torch.Tensor]:
     fastdllm_engine.py:496-503).  The reference lays them out block-diagonally (utils/context.py:73-98); so does
     this, on the active columns only.  The cached context is always visible to the HIP kernels -- it is in every
     mask the reference builds -- so a mask that hides a context column is refused."""
-    parts, all_visible = [], True
+    parts, ctx_ok, act_ok = [], [], []
     for m in masks:
         m = m.reshape(m.shape[-2], m.shape[-1]).to(torch.bool)
         h, w = m.shape
         if w < h:
             raise ValueError(f"sequence mask of {h} rows has only {w} key columns")
-        if w > h and not bool(m[:, :w - h].all()):
-            raise ValueError("a sequence mask hides cached context keys; the HIP attention always sees the "
-                             "visible prefix (pass a shorter context or other ranges instead)")
+        if w > h:
+            ctx_ok.append(m[:, :w - h].all())
         a = m[:, w - h:]
-        all_visible = all_visible and bool(a.all())
+        act_ok.append(a.all())
         parts.append(a)
-    if all_visible:
+    if not parts:
+        return None
+    # one transfer to the host for all sequences: [every context column visible, every active column visible]
+    one = torch.ones((), dtype=torch.bool, device=parts[0].device)
+    flags = torch.stack([torch.stack(ctx_ok).all() if ctx_ok else one, torch.stack(act_ok).all()]).tolist()
+    if not flags[0]:
+        raise ValueError("a sequence mask hides cached context keys; the HIP attention always sees the "
+                         "visible prefix (pass a shorter context or other ranges instead)")
+    if flags[1]:
         return None
     n = sum(p.shape[0] for p in parts)
     out = torch.zeros((n, n), dtype=torch.bool, device=parts[0].device)
@@ -100,13 +113,13 @@ def set_context_diffusion_lm(is_prefill, cu_seqlens_q=None, cu_seqlens_k=None, m
                              slot_mapping=None, context_lens=None, block_tables=None, seqs=None, seq_lens=None,
                              seq_lens_ts=None, kv_cache_layout="unified", need_kv_cache_store=True,
                              decode_delta_state=None, prefill_sparse_state=None, block_mask=None, mask_kind="full",
-                             ranges=None, max_context_len=0) -> None:
+                             ranges=None, max_context_len=0, store_before_attention=False) -> None:
     """Same positional/keyword surface as the reference (context.py:135-152) plus the mask / range
     description the HIP path uses instead of a materialised mask."""
     _THREAD_CONTEXT.diffusion_lm = ContextForDiffusionLM(
         is_prefill, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, slot_mapping, context_lens, block_tables,
         seqs, seq_lens, seq_lens_ts, kv_cache_layout, need_kv_cache_store, block_mask, decode_delta_state,
-        prefill_sparse_state, mask_kind, ranges, max_context_len)
+        prefill_sparse_state, mask_kind, ranges, max_context_len, store_before_attention)
 
 
 def reset_context_diffusion_lm() -> None:

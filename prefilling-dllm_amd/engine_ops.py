@@ -200,27 +200,34 @@ def compact_prompt_cache_per_layer_per_head(kv_cache: torch.Tensor, prompt_page_
 
 def normalize_per_head_keep_indices(keep_indices_per_layer_per_head, *, num_layers: int, num_heads: int,
                                     full_prompt_len: int, device) -> Tuple[List[torch.Tensor], int]:
-    """Shape / range checks of _normalize_per_head_keep_indices (ENG:560-605)."""
-    if len(keep_indices_per_layer_per_head) != num_layers:
-        raise ValueError("per-head keep index layer count mismatch: "
-                         f"got {len(keep_indices_per_layer_per_head)}, expected {num_layers}")
-    normalized: List[torch.Tensor] = []
-    active_len: Optional[int] = None
-    for layer_idx, layer_keep in enumerate(keep_indices_per_layer_per_head):
-        keep = torch.as_tensor(layer_keep, dtype=torch.long, device=device)
-        if keep.ndim != 2:
-            raise ValueError(f"Layer {layer_idx} keep indices must be [num_heads, active_len], got {tuple(keep.shape)}")
-        if int(keep.shape[0]) != num_heads:
-            raise ValueError(f"Layer {layer_idx} keep head count mismatch: got {keep.shape[0]}, expected {num_heads}")
-        if active_len is None:
-            active_len = int(keep.shape[1])
-        elif int(keep.shape[1]) != active_len:
-            raise ValueError(f"Layer {layer_idx} active length mismatch: got {keep.shape[1]}, expected {active_len}")
-        if keep.numel() > 0:
-            if int(keep.min().item()) < 0 or int(keep.max().item()) >= full_prompt_len:
-                raise ValueError(f"Layer {layer_idx} keep indices are outside full prompt length {full_prompt_len}.")
-        normalized.append(keep.contiguous())
-    return normalized, int(active_len or 0)
+    """The contract of _normalize_per_head_keep_indices (ENG:560-605): `num_layers` index tensors
+    [num_heads, active_len] of one common active_len with entries in [0, full_prompt_len); returns them as
+    contiguous int64 tensors on `device` and the active length.  Any violation is a ValueError that names the
+    first offending layer.
+
+    The layers are stacked into one [L, H, n] tensor, so the range check is one pass over all of them and one
+    transfer to the host instead of two per layer."""
+    given = list(keep_indices_per_layer_per_head)
+    if len(given) != num_layers:
+        raise ValueError(f"keep indices for {len(given)} layers were passed, the model has {num_layers}")
+    if num_layers == 0:
+        return [], 0
+    per_layer = [torch.as_tensor(x, dtype=torch.long, device=device) for x in given]
+    shapes = [tuple(t.shape) for t in per_layer]
+    want_tail = shapes[0][1:] if len(shapes[0]) == 2 else None
+    for l, shp in enumerate(shapes):
+        if len(shp) != 2 or shp[0] != num_heads:
+            raise ValueError(f"layer {l}: keep indices have shape {shp}, expected [{num_heads}, active_len]")
+        if shp[1:] != want_tail:
+            raise ValueError(f"layer {l}: {shp[1]} kept tokens per head, layer 0 keeps {want_tail[0]}")
+    stacked = torch.stack(per_layer)                                   # [L, H, n]
+    n_keep = int(stacked.shape[2])
+    if n_keep > 0:
+        bad = ((stacked < 0) | (stacked >= full_prompt_len)).flatten(1).any(dim=1)   # [L]
+        bad_layers = torch.nonzero(bad).flatten().tolist()                          # the one host transfer
+        if bad_layers:
+            raise ValueError(f"layer {bad_layers[0]}: a keep index lies outside the prompt of {full_prompt_len} tokens")
+    return list(stacked.unbind(0)), n_keep
 
 
 def snapshot_prompt_cache_per_layer(kv_cache: torch.Tensor, prompt_page_ids: Sequence[int],

@@ -98,6 +98,9 @@ class PagePool:
     # ---- pages ----
     def allocate_pages(self, n: int) -> List[int]:
         """The n pages that have been free the longest, each with one holder; all or nothing."""
+        n = int(n)
+        if n <= 0:
+            return []          # nothing asked for: no state is touched (the reference returns [] as well, ENG:112-119)
         with self._lock:
             if n > self._n_free:
                 raise RuntimeError(f"Cannot allocate {n} pages, only {self._n_free} free")
@@ -120,9 +123,18 @@ class PagePool:
     def release_pages(self, pages: Sequence[int]) -> None:
         """One holder less per listed page; a page without holders joins the back of the free queue."""
         with self._lock:
-            for p in pages:
-                if self._holders[p] <= 0:
-                    raise RuntimeError(f"page {p} released more often than it was held")
+            # all or nothing: the whole list is checked (a page listed twice needs two holders) before any
+            # count changes, so a refused call leaves the pool as it was
+            listed = np.asarray([int(p) for p in pages], dtype=np.int64)
+            if listed.size == 0:
+                return
+            if listed.min() < 0 or listed.max() >= self._holders.shape[0]:
+                raise RuntimeError(f"page ids {listed.tolist()} are not all pages of this pool")
+            drop = np.bincount(listed, minlength=self._holders.shape[0])
+            over = np.nonzero(drop > self._holders)[0]
+            if over.size:
+                raise RuntimeError(f"page {int(over[0])} released more often than it was held")
+            for p in listed.tolist():
                 self._holders[p] -= 1
                 if self._holders[p] == 0:
                     if self._back == _NIL:
