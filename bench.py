@@ -177,64 +177,152 @@ def _time_us(torch, fn, iters=10, warmup=2, warm_seconds=0.05):
     return e0.elapsed_time(e1) * 1e3 / iters
 
 
-def secondary_shapes(torch, ops, dev):
-    """The other BASELINE configs, one launch (or one layer) each: reported next to the headline number."""
-    out = {}
-    gd = torch.Generator(device=dev).manual_seed(1)
-    std = 1.0 / math.sqrt(D)
+def _graph_us(torch, fn, iters=20):
+    """Device time of fn per call when it is captured once as a HIP graph and replayed: what the launches cost
+    without the host's share (Python, ctypes, allocations) between them."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):       # warm-up on the capture stream (lazy initialisation must not be captured)
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        fn()
+    return _time_us(torch, g.replay, iters)
 
-    # response-only block (the reference engine's real decode shape, 32 rows): the HBM-bound case
+
+def _hbm(by, us):
+    return {"hbm_GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS}
+
+
+def x_decode_32_rows(torch, ops, dev, gd):
+    """Response-only block (the reference engine's real decode shape, 32 rows): the HBM-bound case."""
     w32 = build_workload(torch, dev, q_len=32, layers=4)
     p32 = prepare(ops, w32)
     _, g32 = time_steps(torch, p32, 32, 200)   # 200 warm-up steps of 4 layers = 40 ms: the clocks are up again
     b32, f32_ = algorithmic_work(32, w32["ctx"], w32["n_req"])
     l32 = g32 / (32 * 4)
-    out["decode_32_rows"] = {"us_per_launch": l32 * 1e6, "us_per_step_28_layers": l32 * 28e6,
-                             "hbm_GBps": b32 / l32 / 1e9, "hbm_frac": b32 / l32 / 1e9 / PEAK_HBM_GBS,
-                             "bf16_TFLOPs": f32_ / l32 / 1e12}
-    del w32, p32
+    return {"us_per_launch": l32 * 1e6, "us_per_step_28_layers": l32 * 28e6, "hbm_GBps": b32 / l32 / 1e9,
+            "hbm_frac": b32 / l32 / 1e9 / PEAK_HBM_GBS, "bf16_TFLOPs": f32_ / l32 / 1e12,
+            "plan": p32[0].attn.describe_plan()}
 
-    # configs[3]: chunked BOS-prefixed prefill, 32 chunks x 1025 rows, causal inside a chunk, with the paged
-    # store of K/V (one layer; a prefill is 28 of these)
+
+def _prefill_inputs(torch, ops, dev, gd):
+    """configs[3]: 32 chunks x (1 BOS + 1024) tokens, Q/K/V drawn N(0,1), a seeded page table."""
     L, NC = 1025, 32
     n = L * NC
-    q = (torch.randn((n, HQ, D), generator=gd, device=dev) * std).to(torch.bfloat16)
-    k = (torch.randn((n, HKV, D), generator=gd, device=dev) * std).to(torch.bfloat16)
-    v = (torch.randn((n, HKV, D), generator=gd, device=dev) * std).to(torch.bfloat16)
-    o = torch.empty_like(q)
+    q = torch.randn((n, HQ, D), generator=gd, device=dev).to(torch.bfloat16)
+    k = torch.randn((n, HKV, D), generator=gd, device=dev).to(torch.bfloat16)
+    v = torch.randn((n, HKV, D), generator=gd, device=dev).to(torch.bfloat16)
     pages = (n + PAGE - 1) // PAGE
     kc = torch.zeros((pages + 1, PAGE, HKV, D), dtype=torch.bfloat16, device=dev)
     vc = torch.zeros_like(kc)
     page_ids = torch.randperm(pages, generator=torch.Generator().manual_seed(2)).to(torch.int32).to(dev)
     slots = ops.slot_mapping_from_pages(page_ids, n)
     cu = torch.arange(0, n + 1, L, dtype=torch.int32, device=dev)
+    return L, NC, q, k, v, kc, vc, slots, cu
+
+
+def x_prefill(torch, ops, dev, gd):
+    """configs[3]: chunked BOS-prefixed prefill, causal inside a chunk, with the paged store of K/V (one layer;
+    a prefill is 28 of these)."""
+    L, NC, q, k, v, kc, vc, slots, cu = _prefill_inputs(torch, ops, dev, gd)
+    o = torch.empty_like(q)
     us = _time_us(torch, lambda: ops.chunk_prefill_attention(q, k, v, cu, max_seqlen=L, causal=True, k_cache=kc,
                                                              v_cache=vc, slot_mapping=slots, out=o), 5, 1)
     fl = 2.0 * NC * L * L * D * HQ
-    out["prefill_32x1025_causal_layer"] = {"us_per_layer": us, "bf16_TFLOPs": fl / us / 1e6,
-                                           "mfma_frac": fl / us / 1e6 / PEAK_BF16_TFLOPS,
-                                           "us_per_prefill_28_layers": us * 28}
-    del q, k, v, o, kc, vc
+    return {"us_per_layer": us, "bf16_TFLOPs": fl / us / 1e6, "mfma_frac": fl / us / 1e6 / PEAK_BF16_TFLOPS,
+            "us_per_prefill_28_layers": us * 28, "inputs": "N(0,1)"}
 
-    # configs[1]: draft self-information scores of 32 chunks x 4 labels over a 152064 vocabulary + top-4,
-    # and the column-sum eviction scores of 8 chunks (28 heads x 64 queries x 1025 keys fp32) + keep 256
+
+def x_rope_qk_store(torch, ops, dev, gd):
+    """Rotary embedding of Q and K and the paged store of rotated K and V of the configs[3] layer in one launch
+    (layers/rotary_embedding.py:39-65 + kv_cache_kernels.py:150-172).  Bytes: Q read and written, K and V read,
+    K and V written to the pages."""
+    L, NC, q, k, v, kc, vc, slots, cu = _prefill_inputs(torch, ops, dev, gd)
+    n = L * NC
+    pos = torch.arange(n, device=dev)
+    inv = 1.0 / (1e6 ** (torch.arange(0, D, 2, device=dev).float() / D))
+    ang = torch.arange(n, device=dev).float()[:, None] * inv[None, :]
+    cs = torch.cat([ang.cos(), ang.sin()], dim=-1)
+    us = _time_us(torch, lambda: ops.rope_qk_store(q, k, v, pos, cs, kc, vc, slots), 5, 1)
+    by = n * (2 * HQ * D * 2 + 2 * 2 * HKV * D * 2 + 2 * HKV * D * 2)  # q r+w, k r+w(in place) + v r, pages w
+    return {"us_per_layer": us, **_hbm(by, us)}
+
+
+def x_score(torch, ops, dev, gd):
+    """configs[1]: draft self-information scores of 32 chunks x 4 labels over a 152064 vocabulary + top-4."""
     V2 = 152064
     logits = (torch.randn((32, 4, V2), generator=gd, device=dev) * 2.0).to(torch.bfloat16)
     labels = torch.randint(0, V2, (32, 4), generator=gd, device=dev)
-    us = _time_us(torch, lambda: ops.chunk_select_from_logits(logits, labels, 4))
+    fn = lambda: ops.chunk_select_from_logits(logits, labels, 4)
+    us = _time_us(torch, fn)
     by = logits.numel() * 2
-    out["score_32x4x152064_top4"] = {"us": us, "hbm_GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS}
-    probs = torch.softmax(torch.randn((8, HQ, 64, 1025), generator=gd, device=dev), dim=-1)
-    us = _time_us(torch, lambda: ops.topb_keep_bos(ops.evict_colsum(probs).reshape(8, 1025), 256))
-    by = probs.numel() * 4
-    out["evict_8x28x64x1025_keep256"] = {"us": us, "hbm_GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS}
-    del logits, probs
+    return {"us": us, **_hbm(by, us), "us_graph_replay": _graph_us(torch, fn)}
 
-    # configs[4]: confidence + argmax over [4 x 32, 126464] logits and the threshold-0.9 unmask decision
+
+def x_evict(torch, ops, dev, gd):
+    """configs[1]: column-sum eviction scores of 8 chunks (28 heads x 64 queries x 1025 keys fp32) + keep 256."""
+    probs = torch.softmax(torch.randn((8, HQ, 64, 1025), generator=gd, device=dev), dim=-1)
+    fn = lambda: ops.evict_keep_from_probs(probs, 256)
+    us = _time_us(torch, fn)
+    by = probs.numel() * 4
+    return {"us": us, **_hbm(by, us), "us_graph_replay": _graph_us(torch, fn)}
+
+
+def x_evict_qk(torch, ops, dev, gd):
+    """The eviction scorer from q and k (triton_eviction_scorer.py:114-210) at the reference's shape: 28 heads,
+    the last Lq = 8 / 64 query rows over prefix + 1025-token chunk + queries, causal.  Bytes: K of every visible
+    key once per pass over it (the scorer makes two: row maxima and sums, then the chunk columns) + Q."""
+    out = {}
+    for lq, prefix in ((8, 0), (64, 0), (8, 4096)):
+        n = prefix + 1025 + lq
+        q = (torch.randn((n, HQ, D), generator=gd, device=dev)).to(torch.bfloat16)
+        k = (torch.randn((n, HKV, D), generator=gd, device=dev)).to(torch.bfloat16)
+        fn = lambda: ops.query_to_chunk_attention_scores(q, k, prefix_len=prefix, chunk_len=1025, query_len=lq,
+                                                         scale=D ** -0.5)
+        us = _time_us(torch, fn)
+        by = (n + 1025) * HKV * D * 2 + lq * HQ * D * 2 + HQ * 1025 * 4
+        out[f"Lq{lq}_prefix{prefix}"] = {"us": us, **_hbm(by, us)}
+    return out
+
+
+def x_compact(torch, ops, dev, gd):
+    """Per-head compaction of one configs[2] request (fastdllm_engine.py:607-638): 28 layers x K and V x 4 KV
+    heads, 4096 kept of 32800 prompt tokens gathered and written to the front of the request's pages.  Bytes:
+    the kept rows read and written."""
+    from prefilling_dllm_amd import engine_ops
+    layers, n_tok, kept = LAYERS, 32 * 1025, 4096
+    pages = (n_tok + PAGE - 1) // PAGE
+    kv = torch.randn((2, layers, pages + 1, PAGE, HKV, D), generator=gd, device=dev, dtype=torch.bfloat16)
+    page_ids = torch.randperm(pages, generator=torch.Generator().manual_seed(4)).tolist()
+    g = torch.Generator().manual_seed(5)
+    keep = [torch.stack([torch.randperm(n_tok, generator=g)[:kept].sort().values for _ in range(HKV)]).to(dev)
+            for _ in range(layers)]
+    us = _time_us(torch, lambda: engine_ops.compact_prompt_cache_per_layer_per_head(kv, page_ids, keep), 3, 1)
+    by = 2 * layers * HKV * kept * D * 2 * 2
+    return {"us_per_request": us, **_hbm(by, us)}
+
+
+def x_copy_pages(torch, ops, dev, gd):
+    """Page-granular cache-to-cache copy of one request's prompt KV (fastdllm_engine.py:845-859 as pages): 129
+    pages x 28 layers x K and V, one launch.  Bytes: the pages read and written."""
+    layers, pages = LAYERS, (32 * 1025 + PAGE - 1) // PAGE
+    src = torch.randn((2, layers, pages + 3, PAGE, HKV, D), generator=gd, device=dev, dtype=torch.bfloat16)
+    dst = torch.zeros_like(src)
+    sp = torch.randperm(pages + 3, generator=torch.Generator().manual_seed(6))[:pages].to(torch.int32).to(dev)
+    dp = torch.randperm(pages + 3, generator=torch.Generator().manual_seed(7))[:pages].to(torch.int32).to(dev)
+    us = _time_us(torch, lambda: ops.kv_copy_pages(src, dst, sp, dp), 5, 1)
+    by = 2 * 2 * layers * pages * PAGE * HKV * D * 2
+    return {"us_per_request": us, **_hbm(by, us)}
+
+
+def x_unmask(torch, ops, dev, gd):
+    """configs[4]: confidence + argmax over [4 x 32, 126464] logits and the threshold-0.9 unmask decision."""
     V5 = 126464
     lg = (torch.randn((128, V5), generator=gd, device=dev) * 3.0).to(torch.bfloat16)
     ids = torch.full((4, 32), V5 - 1, dtype=torch.int64, device=dev)
-
     prepared_unmask = ops.PreparedDenoiseUnmask(lg, ids, V5 - 1, 0.9)
 
     def unmask():
@@ -242,17 +330,27 @@ def secondary_shapes(torch, ops, dev):
         prepared_unmask.run()
     us = _time_us(torch, unmask)
     by = lg.numel() * 2
-    out["unmask_4x32x126464"] = {"us": us, "hbm_GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS}
-    del lg
+    return {"us": us, **_hbm(by, us), "us_graph_replay": _graph_us(torch, unmask)}
 
-    # configs[4]: fp8 e4m3 KV pages with a per-page scale, MHA 32/32, 4 requests x 16 chunks x 1025 tokens, 160 rows
+
+def x_fp8(torch, ops, dev, gd):
+    """configs[4]: fp8 e4m3 KV pages with a per-page fp32 scale, MHA 32/32, 4 requests x 16 of 64 chunks x 1025
+    tokens, 160 rows.  The pages hold N(0,1)/sqrt(128) values quantised page by page with scale = amax / 448, as
+    the quantising store writes them."""
     Hm, n_req, ctx5, ql = 32, 4, 16 * 1025, 160
+    std = 1.0 / math.sqrt(D)
     ppr = 64 * 1025 // PAGE + 1
     n_pages = n_req * ppr + 1
-    kc8 = torch.randint(0, 0x78, (n_pages, PAGE, Hm, D), dtype=torch.uint8, device=dev, generator=gd)
-    vc8 = torch.randint(0, 0x78, (n_pages, PAGE, Hm, D), dtype=torch.uint8, device=dev, generator=gd)
-    ks = torch.full((n_pages,), 1.0 / 448, dtype=torch.float32, device=dev)
-    vs = torch.full((n_pages,), 1.0 / 448, dtype=torch.float32, device=dev)
+    kc8 = torch.empty((n_pages, PAGE, Hm, D), dtype=torch.uint8, device=dev)
+    vc8 = torch.empty_like(kc8)
+    ks = torch.empty((n_pages,), dtype=torch.float32, device=dev)
+    vs = torch.empty_like(ks)
+    for cache, scale in ((kc8, ks), (vc8, vs)):
+        for p0 in range(0, n_pages, 64):       # in slabs, to bound the fp32 temporary
+            x = torch.randn((min(64, n_pages - p0), PAGE, Hm, D), generator=gd, device=dev) * std
+            sc = x.abs().amax(dim=(1, 2, 3)) / 448.0
+            scale[p0:p0 + x.shape[0]] = sc
+            cache[p0:p0 + x.shape[0]] = (x / sc.view(-1, 1, 1, 1)).to(torch.float8_e4m3fn).view(torch.uint8)
     bt = torch.arange(n_req * ppr, dtype=torch.int32, device=dev).view(n_req, ppr)
     g = torch.Generator().manual_seed(3)
     ptr, start, length = [0], [], []
@@ -273,9 +371,36 @@ def secondary_shapes(torch, ops, dev):
     us = _time_us(torch, pr.run, 5, 1)
     by = n_req * (2 * ctx5 * Hm * D * 1 + 2 * ql * Hm * D * 2 + 2 * ql * Hm * D * 2)
     fl = n_req * 4.0 * ql * (ctx5 + ql) * D * Hm
-    out["decode_fp8_kv_4x16x1025_mha32_layer"] = {"us_per_layer": us, "hbm_GBps": by / us / 1e3,
-                                                  "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS,
-                                                  "bf16_TFLOPs": fl / us / 1e6}
+    return {"us_per_layer": us, **_hbm(by, us), "bf16_TFLOPs": fl / us / 1e6,
+            "mfma_frac": fl / us / 1e6 / PEAK_BF16_TFLOPS, "plan": pr.describe_plan()}
+
+
+# name in the JSON line -> (short name for --only, function)
+EXTRAS = collections.OrderedDict([
+    ("decode_32_rows", ("decode32", x_decode_32_rows)),
+    ("prefill_32x1025_causal_layer", ("prefill", x_prefill)),
+    ("rope_qk_store_32x1025_layer", ("rope", x_rope_qk_store)),
+    ("score_32x4x152064_top4", ("score", x_score)),
+    ("evict_8x28x64x1025_keep256", ("evict", x_evict)),
+    ("evict_score_qk_28_heads_chunk_1025", ("evictqk", x_evict_qk)),
+    ("compact_per_head_28_layers_4096_of_32800", ("compact", x_compact)),
+    ("kv_copy_pages_129_pages_28_layers", ("copypages", x_copy_pages)),
+    ("unmask_4x32x126464", ("unmask", x_unmask)),
+    ("decode_fp8_kv_4x16x1025_mha32_layer", ("fp8", x_fp8)),
+])
+
+
+def secondary_shapes(torch, ops, dev, only=None):
+    """The other BASELINE configs and the operators around them, one launch (or one layer) each: reported next to
+    the headline number.  `only`: short names to run (the rest is skipped)."""
+    out = {}
+    for name, (short, fn) in EXTRAS.items():
+        if only is not None and short not in only:
+            continue
+        gd = torch.Generator(device=dev).manual_seed(1)
+        out[name] = fn(torch, ops, dev, gd)
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
     return out
 
 
@@ -289,6 +414,10 @@ def main():
     ap.add_argument("--tiles-per-wg", type=int, default=0, help="override the tiles per workgroup (tuning)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary shapes")
+    ap.add_argument("--only", default="", metavar="NAMES",
+                    help="run only these secondary shapes (comma-separated short names: "
+                         + ", ".join(v[0] for v in EXTRAS.values()) + ") and print their results; the headline "
+                         "step is not run (for profiling one kernel)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run a plain device copy of this many MiB (a kernel of known traffic, used to "
                          "scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -314,6 +443,15 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if args.only:
+        only = set(args.only.split(","))
+        unknown = only - {v[0] for v in EXTRAS.values()}
+        if unknown:
+            print(f"bench.py: unknown shape(s) {sorted(unknown)}", file=sys.stderr)
+            sys.exit(2)
+        print(json.dumps({"extras": secondary_shapes(torch, ops, dev, only)}))
+        return
 
     w = build_workload(torch, dev)
     preps = prepare(ops, w, args.rows_per_group, args.num_splits, args.tiles_per_wg)

@@ -159,12 +159,19 @@ class Attention(nn.Module):
         """The layer's full prompt K/V [S, Hkv, d] as pages of a cache of its own (where the reference concatenates,
         attention_v4.py:120-125) with room for `extra` more tokens.  The copy lives in the state between steps and
         is tied to the prompt tensor *objects* it was made from (the entry holds them, so their storage cannot be
-        freed and handed to another tensor while the copy is in use); a caller that rewrites those tensors in place
-        drops the copy with `state.pop("_paged_prompt", None)` or bumps `state["prompt_generation"]`.  The copy
-        doubles the prompt K/V of the layer in device memory for as long as the state lives."""
+        freed and handed to another tensor while the copy is in use) and to their version counters, so an in-place
+        update of the prompt tensors makes a new copy.  Tensors made under torch.inference_mode() -- the reference
+        builds full_k / full_v there (fastdllm_engine.py:656-662) -- have no version counter: a caller that
+        rewrites those in place bumps `state["prompt_generation"]`.  The copy doubles the prompt K/V of the layer in
+        device memory for as long as the state lives."""
         page, n_prompt = 256, int(full_k.shape[0])
         pages = (n_prompt + extra + page - 1) // page
-        generation = state.get("prompt_generation", 0)
+        def version(t):
+            try:
+                return t._version
+            except RuntimeError:      # inference tensors do not track a version counter
+                return -1
+        generation = (state.get("prompt_generation", 0), version(full_k), version(full_v))
         held = state.setdefault("_paged_prompt", {})
         ent = held.get(self.layer_idx)
         fresh = (ent is not None and ent["k"] is full_k and ent["v"] is full_v and ent["n"] == n_prompt

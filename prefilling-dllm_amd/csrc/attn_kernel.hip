@@ -49,6 +49,9 @@
 namespace pdllm {
 
 int launch_attn_fwd2(const AttnKParams& p, int grid, int dyn_lds, bool buf, hipStream_t stream);  // attn_kernel2.hip
+// attn_prefill.hip: resident workgroups that walk a stream of tiles through all their columns (large prefills)
+bool prefill_stream_plan(const pdllm_attn_desc* d, int cus, int* grid, int* team);
+int launch_prefill_stream(const pdllm_attn_desc* d, int grid, int team, hipStream_t stream);
 
 int kv_store_launch(const void* key, const void* value, void* k_cache, void* v_cache,
                     const int32_t* slot_mapping, int64_t n_tokens, int64_t row_elems,
@@ -1561,6 +1564,10 @@ static int launch_slot_table(const AttnKParams& p, int n_req, int* table, hipStr
 static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t stream) {
   int st = validate_desc(d, prefill);
   if (st != PDLLM_OK) return st;
+  if (prefill) {
+    int grid = 0, team = 0;
+    if (prefill_stream_plan(d, compute_units(), &grid, &team)) return launch_prefill_stream(d, grid, team, stream);
+  }
   const AttnPlan plan = make_plan(d, prefill);
   const int64_t need = ws_bytes_for(d, plan.max_pieces, prefill);
   if (need > 0 && (!d->workspace || d->workspace_bytes < need)) return PDLLM_ERR_WORKSPACE;
@@ -1756,6 +1763,13 @@ extern "C" int pdllm_attn_plan_describe(const pdllm_attn_desc* desc, int32_t pre
   const int st = pdllm::validate_desc(desc, prefill != 0);
   if (st != PDLLM_OK) return st;
   if (text == nullptr || text_bytes <= 0) return PDLLM_ERR_NULL;
+  if (prefill) {
+    int grid = 0, team = 0;
+    if (pdllm::prefill_stream_plan(desc, pdllm::compute_units(), &grid, &team)) {
+      const int n = snprintf(text, (size_t)text_bytes, "attn_prefill_stream_kernel kv=bf16 row_blocks=4 grid=%d team=%d", grid, team);
+      return n > 0 && n < text_bytes ? PDLLM_OK : PDLLM_ERR_SHAPE;
+    }
+  }
   const pdllm::AttnPlan plan = pdllm::make_plan(desc, prefill != 0);
   const bool fp8 = !prefill && desc->k_cache != nullptr && desc->max_ctx_len > 0 && desc->kv_dtype == PDLLM_KV_FP8_E4M3;
   const char* kernel = plan.J == 8 && !fp8 ? "attn_fwd2_kernel" : "attn_fwd_kernel";

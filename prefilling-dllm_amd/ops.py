@@ -414,11 +414,13 @@ def chunk_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, c
                             max_seqlen: int, causal: bool = True, sm_scale: Optional[float] = None,
                             k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
                             slot_mapping: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                            rows_per_group: int = 0) -> torch.Tensor:
+                            rows_per_group: int = 0, num_splits: int = 0) -> torch.Tensor:
     """Block-diagonal self-attention over a packed batch of independent chunks
     (attention_v4.py:336-367 with the block mask of utils/context.py:73-84), causal or full
     inside each chunk, with the paged store of K/V (kv_cache_kernels.py:150-172) when
-    slot_mapping is given."""
+    slot_mapping is given.  num_splits = 0 lets the library choose the kernel (resident workgroups that stream
+    through their columns for large batches, one workgroup per column otherwise); 1 asks for one workgroup per
+    column."""
     _need_cuda(q, k, v, cu_seqlens)
     n_tokens, Hq, d = q.shape
     if sm_scale is None:
@@ -428,7 +430,7 @@ def chunk_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, c
     cu = cu_seqlens.to(torch.int32).contiguous()
     mode = _lib.MASK_CAUSAL if causal else _lib.MASK_FULL
     desc = _fill_desc(q, k, v, out, None, None, None, cu, None, None, mode, max_seqlen, 0, sm_scale, None, None,
-                      1, rows_per_group)
+                      num_splits, rows_per_group)
     slots_ptr = None
     if slot_mapping is not None:
         if k_cache is None or v_cache is None:
@@ -444,6 +446,26 @@ def chunk_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, c
         desc.kv_dtype = _lib.KV_BF16
     check(lib.pdllm_chunk_prefill_attn(C.byref(desc), slots_ptr, _stream(q)), "chunk_prefill_attention")
     return out
+
+
+def describe_prefill_plan(n_chunks: int, num_q_heads: int, num_kv_heads: int, max_seqlen: int, n_tokens: int,
+                          causal: bool = True, num_splits: int = 0) -> str:
+    """The launch pdllm_chunk_prefill_attn would make for such a batch, as pdllm_attn_plan_describe words it
+    (which kernel, grid, team or split).  Needs no device memory."""
+    desc = AttnDesc()
+    desc.q = desc.k_new = desc.v_new = desc.out = desc.q_start_loc = 16   # non-NULL, aligned; never dereferenced
+    d = 128
+    desc.q_stride = desc.o_stride = num_q_heads * d
+    desc.kn_stride = desc.vn_stride = num_kv_heads * d
+    desc.n_tokens, desc.n_req = int(n_tokens), int(n_chunks)
+    desc.num_q_heads, desc.num_kv_heads, desc.head_dim = num_q_heads, num_kv_heads, d
+    desc.max_q_len, desc.max_ctx_len = int(max_seqlen), 0
+    desc.mask_mode = _lib.MASK_CAUSAL if causal else _lib.MASK_FULL
+    desc.sm_scale = 1.0 / math.sqrt(d)
+    desc.num_splits = int(num_splits)
+    text = C.create_string_buffer(256)
+    check(lib.pdllm_attn_plan_describe(C.byref(desc), 1, text, 256), "describe_prefill_plan")
+    return text.value.decode()
 
 
 def diffusion_lm_parallel_flash_decoding(query, key, value, output, kv_cache_dtype, key_cache, value_cache,
@@ -575,6 +597,16 @@ def evict_colsum(probs: torch.Tensor, heads_per_group: Optional[int] = None) -> 
     check(lib.pdllm_evict_colsum(probs.data_ptr(), c, h, nq, nk, hpg, _ptr(ws), 0 if ws is None else ws.numel(),
                                  out.data_ptr(), _stream(probs)), "evict_colsum")
     return out
+
+
+def evict_keep_from_probs(probs: torch.Tensor, capacity: int, heads_per_group: Optional[int] = None,
+                          keep_high: bool = True, force_keep_first: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One eviction step from ready-made attention probabilities: evict_colsum followed by topb_keep_bos
+    (fastdllm_engine.py:1230-1322 summed over queries and heads, then :903-927).  probs [chunks, H, Q, K] fp32 ->
+    (scores [chunks, groups, K] fp32, keep indices [chunks * groups, keep] int64, ascending)."""
+    scores = evict_colsum(probs, heads_per_group)
+    c, g, nk = scores.shape
+    return scores, topb_keep_bos(scores.view(c * g, nk), capacity, keep_high, force_keep_first)
 
 
 def query_to_chunk_attention_scores(q: torch.Tensor, k: torch.Tensor, *, prefix_len: int, chunk_len: int,

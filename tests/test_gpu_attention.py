@@ -297,6 +297,38 @@ def test_chunk_prefill_block_diagonal(dev, causal):
     assert torch.equal(kc.cpu(), kc_ref) and torch.equal(vc.cpu(), vc_ref)
 
 
+@pytest.mark.parametrize("lens,heads,causal", [
+    ([300] * 8, (28, 4), True), ([300] * 8, (28, 4), False),
+    ([1025, 700, 64, 1, 333, 1024, 1000, 129] * 2, (28, 4), True),        # ragged: empty columns, single-tile columns
+    ([1025, 700, 64, 1, 333, 1024, 1000, 129] * 2, (28, 4), False),
+    ([2000, 1950], (32, 32), True),                                        # MHA: a column spans two to three key tiles
+    ([4100] * 2, (28, 4), True),                                           # few units: teams of 64 workgroups
+])
+def test_chunk_prefill_stream_kernel(dev, lens, heads, causal):
+    """Large batches of chunks run on resident workgroups that stream through their columns
+    (attn_prefill_stream_kernel); one workgroup per column (num_splits = 1) is the same arithmetic in the same
+    order: the two must agree bit for bit on every row, and with the oracle within the attention bound."""
+    from prefilling_dllm_amd._lib import AttnDesc  # noqa: F401  (the library is loaded)
+    ops = _ops()
+    Hq, Hkv = heads
+    gen = torch.Generator().manual_seed(len(lens) * 131 + Hq + int(causal))
+    n, dd = sum(lens), 128
+    q = torch.randn(n, Hq, dd, generator=gen).to(torch.bfloat16)
+    k = torch.randn(n, Hkv, dd, generator=gen).to(torch.bfloat16)
+    v = torch.randn(n, Hkv, dd, generator=gen).to(torch.bfloat16)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    a = ops.chunk_prefill_attention(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), max_seqlen=max(lens), causal=causal)
+    b = ops.chunk_prefill_attention(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), max_seqlen=max(lens), causal=causal,
+                                    num_splits=1)
+    torch.cuda.synchronize()
+    assert "attn_prefill_stream_kernel" in ops.describe_prefill_plan(len(lens), Hq, Hkv, max(lens), n, causal)
+    assert "attn_fwd_kernel" in ops.describe_prefill_plan(len(lens), Hq, Hkv, max(lens), n, causal, num_splits=1)
+    assert torch.equal(a, b)
+    if n * Hq <= 16 * 1100 * 28 and max(lens) <= 2000:        # the oracle in a few seconds
+        ref = ref_ops.chunk_prefill_attention(q, k, v, cu, causal=causal)
+        check(a.float().cpu(), ref, tol=3e-2)
+
+
 def test_permuting_pages_leaves_output_unchanged(dev):
     """Size-independent property: the physical page order is irrelevant (same logical tokens)."""
     case = configs.chunked_prefix_case(13, n_req=1, n_chunks=4, chunk_tokens=512, topk=4, q_len=32)

@@ -137,11 +137,11 @@ def test_decode_delta_layer(dev, state):
                 .view(block, Hq, d).float().cpu()
         finally:
             reset_context_diffusion_lm()
-    held = st["_paged_prompt"][1][1]
-    assert torch.equal(again(), got) and st["_paged_prompt"][1][1] is held
+    held = st["_paged_prompt"][1]["kc"]
+    assert torch.equal(again(), got) and st["_paged_prompt"][1]["kc"] is held
     st["full_v"][1].mul_(-1.0)
     ref_neg = ref_ops.decode_delta(base, q.float(), k.float(), v.float(), fk.float(), -fv.float(), state)
-    assert (again() - ref_neg).abs().max() <= 3e-2 and st["_paged_prompt"][1][1] is not held
+    assert (again() - ref_neg).abs().max() <= 3e-2 and st["_paged_prompt"][1]["kc"] is not held
     st["full_v"][1].mul_(-1.0)
     # disabled or without a prompt for this layer: the plain decode result
     for off in (dict(st, enabled=False), dict(st, full_k=[None, None])):
@@ -153,6 +153,49 @@ def test_decode_delta_layer(dev, state):
         finally:
             reset_context_diffusion_lm()
         assert (plain.view(block, Hq, d).float().cpu() - base).abs().max() <= 2e-2
+
+
+def test_decode_delta_layer_under_inference_mode(dev):
+    """The reference builds full_k / full_v under torch.inference_mode() (fastdllm_engine.py:656-662) and runs the
+    layer there: inference tensors have no version counter, the layer must not ask for one."""
+    from prefilling_dllm_amd.context import set_context_diffusion_lm, reset_context_diffusion_lm
+    gen = torch.Generator().manual_seed(11)
+    Hq, Hkv, d, P = 28, 4, 128, 256
+    prompt, block = 300, 32
+    mk = lambda n, h, std=1.0: (torch.randn(n, h, d, generator=gen) * std).to(torch.bfloat16)
+    fk, fv = mk(prompt, Hkv, 1.5), mk(prompt, Hkv, 0.2)
+    q, k, v = mk(block, Hq, 2.0), mk(block, Hkv, 1.5), mk(block, Hkv, 0.2)
+    pages = (prompt + P - 1) // P
+    kc = torch.zeros(pages + 1, P, Hkv, d, dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    kc.view(-1, Hkv, d)[:prompt] = fk
+    vc.view(-1, Hkv, d)[:prompt] = fv
+    ranges = [[(c * 64, 64) for c in range(0, prompt // 64, 2)]]
+    rp = torch.tensor([0, len(ranges[0])], dtype=torch.int32)
+    rs = torch.tensor([a for a, _ in ranges[0]], dtype=torch.int32)
+    rl = torch.tensor([b for _, b in ranges[0]], dtype=torch.int32)
+    bt = torch.arange(pages + 1, dtype=torch.int32).view(1, -1)
+    cu = torch.tensor([0, block], dtype=torch.int32)
+    n_ctx = sum(b for _, b in ranges[0])
+    state = dict(enabled=True)
+    layer = _layer(dev, Hq, Hkv, d)
+    layer.k_cache, layer.v_cache = kc.to(dev), vc.to(dev)
+    with torch.inference_mode():
+        st = dict(state, full_k=[None, fk.to(dev).clone()], full_v=[None, fv.to(dev).clone()])
+        assert st["full_k"][1].is_inference()
+        outs = []
+        for _ in range(2):      # the second call reuses the paged copy of the prompt
+            set_context_diffusion_lm(False, cu_seqlens_q=cu.to(dev), max_seqlen_q=block, max_seqlen_k=n_ctx + block,
+                                     block_tables=bt.to(dev), need_kv_cache_store=False, decode_delta_state=st,
+                                     ranges=(rp.to(dev), rs.to(dev), rl.to(dev), len(ranges[0])), max_context_len=n_ctx)
+            try:
+                outs.append(layer(q.to(dev).view(block, -1), k.to(dev).view(block, -1), v.to(dev).view(block, -1))
+                            .view(block, Hq, d).float().cpu())
+            finally:
+                reset_context_diffusion_lm()
+    base = ref_ops.sparse_decode_attention(q, k, v, kc, vc, bt, [0, block], ranges)
+    ref = ref_ops.decode_delta(base, q.float(), k.float(), v.float(), fk.float(), fv.float(), state)
+    assert (outs[0] - ref).abs().max() <= 3e-2 and torch.equal(outs[0], outs[1])
 
 
 @pytest.mark.parametrize("state,selection", [
