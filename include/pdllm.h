@@ -264,11 +264,15 @@ int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t n_heads, in
  * k [S, Hkv, d] bf16 contiguous, S = prefix_len + chunk_len + query_len; for every
  * q-head, softmax over the visible keys of the last query_len rows, summed (or averaged)
  * over those rows on the chunk columns -> out [Hq, chunk_len] fp32.
- * causal != 0: key j visible to row i iff j <= i.  workspace: 2*Hq*query_len floats. */
+ * causal != 0: key j visible to row i iff j <= i.  workspace: pdllm_evict_score_qk_workspace_bytes() bytes
+ * (per-row softmax statistics of the key segments; fp32).  head_dim 128 runs on the matrix cores (QK^T in
+ * bf16 with fp32 accumulation, as the reference's tl.dot), other head dims up to 256 on the vector unit. */
+int64_t pdllm_evict_score_qk_workspace_bytes(int64_t prefix_len, int64_t chunk_len, int64_t query_len,
+                                             int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim);
 int pdllm_evict_score_qk(const void* q, const void* k, int64_t prefix_len, int64_t chunk_len,
                          int64_t query_len, int32_t num_q_heads, int32_t num_kv_heads,
                          int32_t head_dim, float scale, int32_t reduce_mean, int32_t causal,
-                         float* workspace, float* out, pdllm_stream_t stream);
+                         float* workspace, int64_t workspace_bytes, float* out, pdllm_stream_t stream);
 
 /* Replaces the pooling + per-KV-head grouping of ENG:1405-1433: optional max/avg pool
  * (kernel, padding kernel/2, stride 1, as F.max_pool1d / F.avg_pool1d with

@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libpdllm_hip.so")
+# (PDLLM_LIB names another build of the same library, e.g. to compare two kernel versions in one session)
+LIB_PATH = os.environ.get("PDLLM_LIB") or os.path.join(_HERE, "libpdllm_hip.so")
 
 PDLLM_OK = 0
 ERRORS = {
@@ -72,7 +73,8 @@ SIGNATURES = {
     "pdllm_topk_lowest_index": (C.c_int, [vp, i64, i64, i64, i64, i32, vp, vp]),
     "pdllm_evict_colsum": (C.c_int, [vp, i64, i64, i64, i64, i64, vp, i64, vp, vp]),
     "pdllm_evict_colsum_workspace_bytes": (i64, [i64, i64, i64]),
-    "pdllm_evict_score_qk": (C.c_int, [vp, vp, i64, i64, i64, i32, i32, i32, f32, i32, i32, vp, vp, vp]),
+    "pdllm_evict_score_qk_workspace_bytes": (i64, [i64, i64, i64, i32, i32, i32]),
+    "pdllm_evict_score_qk": (C.c_int, [vp, vp, i64, i64, i64, i32, i32, i32, f32, i32, i32, vp, i64, vp, vp]),
     "pdllm_token_score_pool_group": (C.c_int, [vp, i64, i64, i32, i32, i64, vp, vp]),
     "pdllm_topb_keep_bos": (C.c_int, [vp, i64, i64, i64, i64, i32, i32, vp, vp]),
     "pdllm_kv_gather": (C.c_int, [vp, vp, i64, vp, i64, i64, i64, i32, i32, i32, i64, i32, vp, vp]),

@@ -16,4 +16,4 @@ extern "C" const char* pdllm_status_string(int status) {
   }
 }
 
-extern "C" int pdllm_abi_version(void) { return 4; }
+extern "C" int pdllm_abi_version(void) { return 5; }

@@ -436,6 +436,10 @@ __global__ __launch_bounds__(256) void pool_group_kernel(const float* __restrict
   out[g * n + i] = hpg > 1 ? acc / (float)hpg : acc;
 }
 
+int evict_score_qk_scalar(const void* q, const void* k, int64_t prefix_len, int64_t chunk_len, int64_t query_len,
+                          int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, float scale, int32_t reduce_mean,
+                          int32_t causal, float* workspace, float* out, hipStream_t stream);
+
 static int topk_launch(const float* scores, int64_t n_rows, int64_t n, int64_t stride, int64_t k,
                        int descending, int force_first, int nonfinite, int sorted_ascending,
                        int64_t* out, hipStream_t stream) {
@@ -531,18 +535,15 @@ extern "C" int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t 
   return launch_status();
 }
 
-extern "C" int pdllm_evict_score_qk(const void* q, const void* k, int64_t prefix_len, int64_t chunk_len,
-                                    int64_t query_len, int32_t num_q_heads, int32_t num_kv_heads,
-                                    int32_t head_dim, float scale, int32_t reduce_mean, int32_t causal,
-                                    float* workspace, float* out, pdllm_stream_t stream) {
-  if (!q || !k || !workspace || !out) return PDLLM_ERR_NULL;
-  if (prefix_len < 0 || chunk_len <= 0 || query_len <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 ||
-      num_q_heads % num_kv_heads || head_dim <= 0)
-    return PDLLM_ERR_SHAPE;
-  if (head_dim > 256 || query_len > 64) return PDLLM_ERR_UNSUPPORTED;  // limits of the reference scorer
+// The eviction scorer on the vector unit, any head dim up to 256 (pdllm_evict_score_qk in evict_qk.hip takes
+// head dim 128 to the matrix cores and everything else here).  workspace: 2 * Hq * query_len floats; the
+// arguments have been checked.
+int pdllm::evict_score_qk_scalar(const void* q, const void* k, int64_t prefix_len, int64_t chunk_len,
+                                 int64_t query_len, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                 float scale, int32_t reduce_mean, int32_t causal, float* workspace, float* out,
+                                 hipStream_t st) {
   float* mx = workspace;
   float* den = workspace + (int64_t)num_q_heads * query_len;
-  hipStream_t st = static_cast<hipStream_t>(stream);
   hipLaunchKernelGGL(evict_maxden_kernel, dim3((unsigned)num_q_heads, (unsigned)query_len), dim3(256), 0, st,
                      static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), (long)prefix_len,
                      (long)chunk_len, (long)query_len, num_q_heads, num_kv_heads, head_dim, scale, causal,

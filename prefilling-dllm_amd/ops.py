@@ -643,10 +643,14 @@ def query_to_chunk_attention_scores(q: torch.Tensor, k: torch.Tensor, *, prefix_
     q = q.to(torch.bfloat16).contiguous()
     k = k.to(torch.bfloat16).contiguous()
     out = torch.empty((hq, int(chunk_len)), device=q.device, dtype=torch.float32)
-    ws = torch.empty(2 * hq * int(query_len), device=q.device, dtype=torch.float32)
+    need = int(lib.pdllm_evict_score_qk_workspace_bytes(prefix_len, chunk_len, query_len, hq, hkv, d))
+    if need < 0:
+        check(need, "query_to_chunk_attention_scores")
+    ws = _workspace(q.device, need)
     check(lib.pdllm_evict_score_qk(q.data_ptr(), k.data_ptr(), prefix_len, chunk_len, query_len, hq, hkv, d,
                                    float(scale), 1 if (reduce_mode or "sum").lower() == "mean" else 0, causal,
-                                   ws.data_ptr(), out.data_ptr(), _stream(q)), "query_to_chunk_attention_scores")
+                                   ws.data_ptr(), ws.numel(), out.data_ptr(), _stream(q)),
+          "query_to_chunk_attention_scores")
     return out
 
 

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(_lib.lib, n), f"{n} declared in pdllm.h but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
-    assert _lib.lib.pdllm_abi_version() == 4
+    assert _lib.lib.pdllm_abi_version() == 5
     assert _lib.lib.pdllm_status_string(0) == b"ok"
 
 

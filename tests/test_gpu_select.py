@@ -155,6 +155,37 @@ def test_query_to_chunk_scores(dev):
                                             query_len=65, scale=scale)
 
 
+@pytest.mark.parametrize("prefix,chunk,ql,Hq,Hkv,d", [
+    (0, 1025, 64, 28, 4, 128), (700, 1025, 8, 28, 4, 128), (5, 130, 1, 28, 4, 128), (33, 257, 20, 8, 8, 128),
+    (0, 64, 13, 32, 2, 128),      # 16 q-heads per KV head
+    (10, 100, 8, 4, 2, 64),       # another head dim: the vector-unit kernels
+])
+def test_query_to_chunk_scores_shapes(dev, prefix, chunk, ql, Hq, Hkv, d):
+    """The matrix-core scorer (head dim 128) and the vector-unit one over ragged shapes: padding rows (query_len
+    not a multiple of 8), several key segments, chunk lengths that are no multiple of 32, causal and full, and
+    the same bits on a second run (fixed order of additions)."""
+    gen = torch.Generator().manual_seed(prefix + chunk + ql)
+    S = prefix + chunk + ql
+    q = torch.randn(S, Hq, d, generator=gen).to(torch.bfloat16)
+    k = torch.randn(S, Hkv, d, generator=gen).to(torch.bfloat16)
+    scale = d ** -0.5
+    ops = _ops()
+    for mask in ("causal", "full"):
+        for red in ("sum", "mean"):
+            kw = dict(prefix_len=prefix, chunk_len=chunk, query_len=ql, scale=scale, reduce_mode=red, attention_mask=mask)
+            got = ops.query_to_chunk_attention_scores(q.to(dev), k.to(dev), **kw).cpu()
+            again = ops.query_to_chunk_attention_scores(q.to(dev), k.to(dev), **kw).cpu()
+            ref = ref_ops.chunk_attention_head_scores(q, k, **kw)
+            assert got.shape == ref.shape == (Hq, chunk)
+            assert (got - ref).abs().max() <= 1e-4 * ref.abs().max() + 1e-7, (mask, red, (got - ref).abs().max())
+            assert torch.equal(got, again)
+    # every key column's mass over all heads and rows: a causal row sees itself, so the chunk columns of a row
+    # never hold all of its mass; a full row's mass over chunk + the rest is 1
+    full = ops.query_to_chunk_attention_scores(q.to(dev), k.to(dev), prefix_len=prefix, chunk_len=chunk, query_len=ql,
+                                               scale=scale, attention_mask="full").cpu()
+    assert (full.sum(dim=1) <= ql + 1e-3).all() and (full >= 0).all()
+
+
 def test_pool_and_group(dev):
     gen = torch.Generator().manual_seed(10)
     s = torch.rand(28, 1025, generator=gen)
