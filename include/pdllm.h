@@ -320,6 +320,20 @@ int pdllm_kv_scatter(void* cache, const int32_t* page_ids, int64_t n_page_ids, i
                      int64_t n_tokens, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
                      int64_t n_pages, int32_t elem_bytes, const void* src, pdllm_stream_t stream);
 
+/* Replaces _compact_prompt_cache_per_layer_per_head (ENG:607-638) for all layers at once: on the unified cache
+ * kv_cache [2, n_layers, n_pages, page_size, Hkv, d] (plane stride in bytes), token j of KV head h of layer l becomes
+ * token keep[l*keep_layer_stride + h*keep_head_stride + j] of the request's pages (page_ids), j < n_keep, for K and V.
+ * The kept rows of a round of layers are gathered into the workspace before the first one is overwritten (the
+ * reference clones), two launches per round; the workspace holds at least one layer
+ * (pdllm_kv_compact_per_head_workspace_bytes) and as many layers per round as fit. */
+int64_t pdllm_kv_compact_per_head_workspace_bytes(int64_t n_keep, int32_t num_kv_heads, int32_t head_dim,
+                                                  int32_t elem_bytes);
+int pdllm_kv_compact_per_head(void* kv_cache, int64_t plane_stride_bytes, int32_t n_layers,
+                              const int32_t* page_ids, int64_t n_page_ids, const int64_t* keep,
+                              int64_t keep_layer_stride, int64_t keep_head_stride, int64_t n_keep,
+                              int32_t num_kv_heads, int32_t head_dim, int32_t page_size, int64_t n_pages,
+                              int32_t elem_bytes, void* workspace, int64_t workspace_bytes, pdllm_stream_t stream);
+
 /* Replaces the per-layer advanced-indexing copies of make_pd_record_from_remote_engine
  * (ENG:845-859) for two unified caches [planes, n_pages, page_size, Hkv, d] (plane = K/V x layer)
  * of the same page geometry: dst[plane][dst_page_ids[i]] = src[plane][src_page_ids[i]] for all

@@ -174,6 +174,52 @@ __global__ __launch_bounds__(256) void kv_scatter_kernel(
   cache[slot * per_tok + rem] = src[idx];
 }
 
+// Per-head compaction of the prompt rows of several planes (K/V x layer) at once: plane y of the launch gathers
+// token keep[layer][head][j] of every head into row j of a dense staging plane, a second launch writes the staged
+// rows to tokens 0 .. n_keep - 1 of the same pages.  Two launches per round of layers, whatever their number
+// (the gather is complete before the first row is overwritten, as in the reference, which clones).
+__global__ __launch_bounds__(256) void kv_compact_gather_kernel(
+    const uint4* __restrict__ cache, long plane16, const int* __restrict__ page_ids, long n_page_ids,
+    const long* __restrict__ keep, long keep_layer_stride, long keep_head_stride, long n_keep, int n_heads,
+    int chunks_per_head, int page_shift, long n_pages, int layer0, int layers_round, int n_layers,
+    uint4* __restrict__ staged) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const long per_tok = (long)n_heads * chunks_per_head;
+  const long j = idx / per_tok;
+  if (j >= n_keep) return;
+  const int rem = (int)(idx - j * per_tok);
+  const int head = rem / chunks_per_head;
+  const int kv = blockIdx.y / layers_round, li = blockIdx.y - kv * layers_round;
+  const long t = keep[(long)(layer0 + li) * keep_layer_stride + (long)head * keep_head_stride + j];
+  uint4 v = {0u, 0u, 0u, 0u};
+  const long pi = t >> page_shift;
+  if (t >= 0 && pi < n_page_ids) {
+    const long page = page_ids[pi];
+    if (page >= 0 && page < n_pages) {
+      const long slot = (page << page_shift) + (t & ((1L << page_shift) - 1));
+      v = cache[((long)kv * n_layers + layer0 + li) * plane16 + slot * per_tok + rem];
+    }
+  }
+  staged[(long)blockIdx.y * n_keep * per_tok + idx] = v;
+}
+
+__global__ __launch_bounds__(256) void kv_compact_scatter_kernel(
+    uint4* __restrict__ cache, long plane16, const int* __restrict__ page_ids, long n_page_ids, long n_keep,
+    long per_tok, int page_shift, long n_pages, int layer0, int layers_round, int n_layers,
+    const uint4* __restrict__ staged) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const long j = idx / per_tok;
+  if (j >= n_keep) return;
+  const int rem = (int)(idx - j * per_tok);
+  const long pi = j >> page_shift;
+  if (pi >= n_page_ids) return;
+  const long page = page_ids[pi];
+  if (page < 0 || page >= n_pages) return;
+  const int kv = blockIdx.y / layers_round, li = blockIdx.y - kv * layers_round;
+  const long slot = (page << page_shift) + (j & ((1L << page_shift) - 1));
+  cache[((long)kv * n_layers + layer0 + li) * plane16 + slot * per_tok + rem] = staged[(long)blockIdx.y * n_keep * per_tok + idx];
+}
+
 // whole pages between two caches, all planes (K/V x layer) in one launch:
 // dst[plane][dst_page_ids[i]] = src[plane][src_page_ids[i]]; pages outside either cache are skipped
 __global__ __launch_bounds__(256) void kv_copy_pages_kernel(
@@ -351,6 +397,55 @@ extern "C" int pdllm_kv_scatter(void* cache, const int32_t* page_ids, int64_t n_
                      (long)n_page_ids, (long)dst_start, (long)n_tokens, per_tok, shift, (long)n_pages,
                      static_cast<const uint4*>(src));
   return launch_status();
+}
+
+extern "C" int64_t pdllm_kv_compact_per_head_workspace_bytes(int64_t n_keep, int32_t num_kv_heads, int32_t head_dim,
+                                                             int32_t elem_bytes) {
+  if (n_keep < 0 || num_kv_heads <= 0 || head_dim <= 0 || (elem_bytes != 1 && elem_bytes != 2)) return PDLLM_ERR_SHAPE;
+  return 2 * n_keep * (int64_t)num_kv_heads * head_dim * elem_bytes;  // K and V of one layer
+}
+
+extern "C" int pdllm_kv_compact_per_head(void* kv_cache, int64_t plane_stride_bytes, int32_t n_layers,
+                                         const int32_t* page_ids, int64_t n_page_ids, const int64_t* keep,
+                                         int64_t keep_layer_stride, int64_t keep_head_stride, int64_t n_keep,
+                                         int32_t num_kv_heads, int32_t head_dim, int32_t page_size, int64_t n_pages,
+                                         int32_t elem_bytes, void* workspace, int64_t workspace_bytes,
+                                         pdllm_stream_t stream) {
+  if (!kv_cache || !page_ids || !keep || !workspace) return PDLLM_ERR_NULL;
+  const int shift = ilog2_exact_l(page_size);
+  if (shift < 0 || n_layers <= 0 || n_page_ids < 0 || n_keep < 0 || num_kv_heads <= 0 || head_dim <= 0 || n_pages <= 0)
+    return PDLLM_ERR_SHAPE;
+  if (elem_bytes != 1 && elem_bytes != 2) return PDLLM_ERR_DTYPE;
+  if (((long)head_dim * elem_bytes) % 16 || plane_stride_bytes % 16) return PDLLM_ERR_STRIDE;
+  if (plane_stride_bytes < n_pages * (int64_t)page_size * num_kv_heads * head_dim * elem_bytes) return PDLLM_ERR_STRIDE;
+  if (!aligned16(kv_cache) || !aligned16(workspace)) return PDLLM_ERR_STRIDE;
+  if (n_keep == 0) return PDLLM_OK;
+  const int64_t per_layer = pdllm_kv_compact_per_head_workspace_bytes(n_keep, num_kv_heads, head_dim, elem_bytes);
+  if (workspace_bytes < per_layer) return PDLLM_ERR_WORKSPACE;
+  int64_t round = workspace_bytes / per_layer;   // layers staged at a time
+  if (round > n_layers) round = n_layers;
+  if (round > 32767) round = 32767;
+  const int cph = head_dim * elem_bytes / 16;
+  const long per_tok = (long)num_kv_heads * cph;
+  const long total = n_keep * per_tok;
+  if ((total + 255) / 256 > 0x7fffffffL) return PDLLM_ERR_SHAPE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  for (int64_t l0 = 0; l0 < n_layers; l0 += round) {
+    const int lr = (int)(n_layers - l0 < round ? n_layers - l0 : round);
+    const dim3 grid((unsigned)((total + 255) / 256), (unsigned)(2 * lr));
+    hipLaunchKernelGGL(kv_compact_gather_kernel, grid, dim3(256), 0, st, static_cast<const uint4*>(kv_cache),
+                       (long)(plane_stride_bytes / 16), page_ids, (long)n_page_ids, reinterpret_cast<const long*>(keep),
+                       (long)keep_layer_stride, (long)keep_head_stride, (long)n_keep, num_kv_heads, cph, shift,
+                       (long)n_pages, (int)l0, lr, n_layers, static_cast<uint4*>(workspace));
+    int rc = launch_status();
+    if (rc != PDLLM_OK) return rc;
+    hipLaunchKernelGGL(kv_compact_scatter_kernel, grid, dim3(256), 0, st, static_cast<uint4*>(kv_cache),
+                       (long)(plane_stride_bytes / 16), page_ids, (long)n_page_ids, (long)n_keep, per_tok, shift,
+                       (long)n_pages, (int)l0, lr, n_layers, static_cast<const uint4*>(workspace));
+    rc = launch_status();
+    if (rc != PDLLM_OK) return rc;
+  }
+  return PDLLM_OK;
 }
 
 extern "C" int pdllm_kv_copy_pages(const void* src_cache, void* dst_cache, const int32_t* src_page_ids,

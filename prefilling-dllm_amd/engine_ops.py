@@ -184,17 +184,21 @@ def compact_prompt_cache_per_head(layer_cache: torch.Tensor, page_ids: torch.Ten
 
 def compact_prompt_cache_per_layer_per_head(kv_cache: torch.Tensor, prompt_page_ids: Sequence[int],
                                             keep_indices_per_layer_per_head: Sequence[torch.Tensor]) -> int:
-    """_compact_prompt_cache_per_layer_per_head (ENG:607-638) on kv_cache [2, L, pages, P, Hkv, d]."""
+    """_compact_prompt_cache_per_layer_per_head (ENG:607-638) on kv_cache [2, L, pages, P, Hkv, d]: all layers, K and
+    V in one library call."""
     if not keep_indices_per_layer_per_head:
         return 0
     page_ids = torch.as_tensor(list(prompt_page_ids), dtype=torch.int32, device=kv_cache.device)
     active_len = int(keep_indices_per_layer_per_head[0].shape[1])
     if active_len <= 0:
         return 0
-    for layer_idx, keep in enumerate(keep_indices_per_layer_per_head):
-        keep = keep.to(device=kv_cache.device, dtype=torch.long)
-        for kv in range(2):
-            compact_prompt_cache_per_head(kv_cache[kv, layer_idx], page_ids, keep)
+    keep = torch.stack([k.to(device=kv_cache.device, dtype=torch.long) for k in keep_indices_per_layer_per_head])
+    if kv_cache.is_contiguous() and keep.shape[0] == kv_cache.shape[1]:
+        ops.kv_compact_per_head(kv_cache, page_ids, keep)
+    else:       # a view of a larger cache, or fewer keep lists than layers: layer by layer
+        for layer_idx in range(keep.shape[0]):
+            for kv in range(2):
+                compact_prompt_cache_per_head(kv_cache[kv, layer_idx], page_ids, keep[layer_idx])
     return active_len
 
 

@@ -746,6 +746,31 @@ def kv_scatter(layer_cache: torch.Tensor, page_ids: torch.Tensor, src: torch.Ten
                                _stream(layer_cache)), "kv_scatter")
 
 
+def kv_compact_per_head(kv_cache: torch.Tensor, page_ids: torch.Tensor, keep: torch.Tensor,
+                        max_workspace_bytes: int = 256 << 20) -> None:
+    """In place on the unified cache kv_cache [2, layers, n_pages, page_size, Hkv, d]: token j of KV head h of
+    layer l <- token keep[l, h, j] of the request's pages, for K and V (fastdllm_engine.py:607-638 for all layers:
+    two launches per round of layers instead of two per layer and tensor).  keep: int64 [layers, Hkv, n_keep]."""
+    _need_cuda(kv_cache, page_ids, keep)
+    if kv_cache.dim() != 6 or not kv_cache.is_contiguous() or kv_cache.shape[0] != 2:
+        raise ValueError("kv_cache must be contiguous [2, layers, n_pages, page_size, Hkv, d]")
+    _, layers, n_pages, P, hkv, d = kv_cache.shape
+    keep = keep.to(torch.int64).contiguous()
+    if keep.dim() != 3 or keep.shape[0] != layers or keep.shape[1] != hkv:
+        raise ValueError(f"keep must be [layers, Hkv, n_keep] = [{layers}, {hkv}, n], got {tuple(keep.shape)}")
+    n_keep = int(keep.shape[2])
+    if n_keep == 0:
+        return
+    page_ids = page_ids.to(torch.int32).contiguous()
+    esz = kv_cache.element_size()
+    per_layer = int(lib.pdllm_kv_compact_per_head_workspace_bytes(n_keep, hkv, d, esz))
+    ws = _workspace(kv_cache.device, min(max(per_layer, int(max_workspace_bytes)), per_layer * layers))
+    check(lib.pdllm_kv_compact_per_head(kv_cache.data_ptr(), kv_cache.stride(1) * esz, layers, page_ids.data_ptr(),
+                                        page_ids.numel(), keep.data_ptr(), keep.stride(0), keep.stride(1), n_keep,
+                                        hkv, d, P, n_pages, esz, ws.data_ptr(), ws.numel(), _stream(kv_cache)),
+          "kv_compact_per_head")
+
+
 def kv_copy_pages(src_kv_cache: torch.Tensor, dst_kv_cache: torch.Tensor, src_page_ids: torch.Tensor,
                   dst_page_ids: torch.Tensor) -> None:
     """dst[:, :, dst_page_ids[i]] = src[:, :, src_page_ids[i]] for two unified caches

@@ -202,6 +202,36 @@ def test_per_head_compaction_matches_reference_order(dev):
     assert torch.equal(dc.cpu(), ref)
 
 
+@pytest.mark.parametrize("sorted_keep,ws_layers", [(True, 3), (False, 1), (True, 99)])
+def test_per_head_compaction_all_layers_in_one_call(dev, sorted_keep, ws_layers):
+    """compact_prompt_cache_per_layer_per_head on a whole cache: K and V of every layer, each KV head with its own
+    keep list, in rounds of as many layers as the workspace holds; unsorted keep lists too (the gather of a round
+    is complete before its first row is overwritten, as in the reference, which clones)."""
+    from prefilling_dllm_amd import engine_ops
+    ops = _ops()
+    gen = torch.Generator().manual_seed(31 + ws_layers)
+    L, n_pages, Hkv, d = 5, 9, 4, 128
+    kv = torch.randn(2, L, n_pages, 256, Hkv, d, generator=gen).to(torch.bfloat16)
+    page_ids = torch.randperm(n_pages, generator=gen)[:6]
+    full_len, keep_n = 1400, 520
+    def one():
+        idx = torch.randperm(full_len, generator=gen)[:keep_n]
+        return torch.sort(idx).values if sorted_keep else idx
+    keeps = [torch.stack([one() for _ in range(Hkv)]) for _ in range(L)]
+    ref = kv.clone()
+    for l in range(L):
+        for which in range(2):
+            ref_ops.compact_per_head(ref[which, l], page_ids, keeps[l])
+    dkv = kv.to(dev)
+    per_layer = 2 * keep_n * Hkv * d * 2
+    ops.kv_compact_per_head(dkv, page_ids.to(dev), torch.stack(keeps).to(dev), max_workspace_bytes=per_layer * ws_layers)
+    torch.cuda.synchronize()
+    assert torch.equal(dkv.cpu(), ref)
+    dkv2 = kv.to(dev)
+    assert engine_ops.compact_prompt_cache_per_layer_per_head(dkv2, page_ids.tolist(), [k.to(dev) for k in keeps]) == keep_n
+    assert torch.equal(dkv2.cpu(), ref)
+
+
 def test_chunk_local_kv_copy_matches_reference_order(dev):
     """fastdllm_engine.py:525-558: the kept tokens of a chunk that was prefilled into temporary pages go, per layer
     and KV head, behind dst_start of the request's pages.  Source chunk and destination both start inside a page,
