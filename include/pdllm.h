@@ -104,9 +104,10 @@ typedef struct pdllm_attn_desc {
   const void* v_cache;
   const float* k_scale; /* fp8 only: scale[page*scale_page_stride + kvh*scale_head_stride] */
   const float* v_scale;
-  const int32_t* block_table; /* [n_req, bt_stride] page ids.  Every page a visible range touches must hold a
-                                 valid id: an entry outside [0, n_pages) is clamped into the cache (never read out
-                                 of bounds), its keys then count like any others */
+  const int32_t* block_table; /* [n_req, bt_stride] page ids.  An entry outside [0, n_pages) (the reference's -1)
+                                 names no page: the keys of a visible range that fall on it are left out, as
+                                 load_kvcache skips such entries (OPS/kv_cache_kernels.py:208).  (Only a request
+                                 whose ranges touch more than 2048 pages has them clamped into the cache instead.) */
   const int32_t* q_start_loc; /* [n_req+1] first active row of each request     */
   /* visible prefix of request r = ranges range_ptr[r] .. range_ptr[r+1]-1, each a
    * run of logical tokens [range_start, range_start+range_len) that is mapped

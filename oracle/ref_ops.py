@@ -190,7 +190,9 @@ def _sdpa(q, k, v, mask, scale, dtype=torch.float32):
 
 def gather_prefix(k_cache, v_cache, block_table_row, ranges, page_size=PAGE_SIZE):
     """Rows of the visible prefix: logical tokens of every (start, len) range mapped through the
-    request's page table (page_table[t // P], t % P) -- the addressing of prefix_prefill.py:100-109."""
+    request's page table (page_table[t // P], t % P) -- the addressing of prefix_prefill.py:100-109.
+    A page-table entry outside [0, n_pages) names no page; its tokens are left out, as load_kvcache skips -1
+    entries (kv_cache_kernels.py:208)."""
     toks: List[int] = []
     for start, length in ranges:
         toks.extend(range(int(start), int(start) + int(length)))
@@ -199,6 +201,8 @@ def gather_prefix(k_cache, v_cache, block_table_row, ranges, page_size=PAGE_SIZE
         return empty, empty.clone()
     t = torch.tensor(toks, dtype=torch.long)
     pages = torch.as_tensor(block_table_row, dtype=torch.long).index_select(0, t // page_size)
+    named = (pages >= 0) & (pages < k_cache.shape[0])
+    pages, t = pages[named], t[named]
     return k_cache[pages, t % page_size], v_cache[pages, t % page_size]
 
 

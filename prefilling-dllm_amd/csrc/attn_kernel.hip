@@ -1091,13 +1091,22 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
 
 // Slot table: for request r and v < count(r), table[r][v] = page * page_size + offset of the v-th
 // visible prefix key (ranges in order, each mapped through the page table); entries up to the
-// next multiple of the tile size repeat the first key of their tile (they are loaded but
-// masked); table[r][stride - 1] = count(r) = min(sum of range lengths, max_ctx_len).
-// Page ids outside [0, n_pages) are clamped, so a slot never points outside the cache.
+// next multiple of the tile size repeat a valid slot (they are loaded but masked);
+// table[r][stride - 1] = count(r).
+// A page-table entry outside [0, n_pages) names no page: its keys are left out, as the reference skips such
+// entries (layers/attention/ops/kv_cache_kernels.py:208), and count(r) is the number of keys that remain, at most
+// max_ctx_len of them.  (A request whose ranges touch more than kMaxSegments pages keeps the older behaviour:
+// such entries are clamped into the cache.)
+constexpr int kMaxSegments = 2048;  // (range, page) pieces of one request's visible prefix
+
 __global__ __launch_bounds__(256) void attn_slot_table_kernel(const AttnKParams p, int* __restrict__ table) {
-  __shared__ int s_cum[kMaxRanges + 1];
+  __shared__ int s_cum[kMaxRanges + 1];      // visible keys before range i, invalid pages included
   __shared__ int s_start[kMaxRanges];
   __shared__ int s_len[kMaxRanges];
+  __shared__ int s_seg0[kMaxRanges + 1];     // pieces before range i
+  __shared__ int s_gone[kMaxSegments];       // keys left out before piece s (exclusive prefix of the invalid pieces' lengths)
+  __shared__ int s_wave[4];
+  __shared__ int s_total_gone;
   const int tid = threadIdx.x;
   const int req = blockIdx.y;
   const int r0 = p.range_ptr[req];
@@ -1110,26 +1119,98 @@ __global__ __launch_bounds__(256) void attn_slot_table_kernel(const AttnKParams 
   }
   __syncthreads();
   if (tid == 0) {
-    int cc = 0;
-    for (int i = 0; i < nr; ++i) { s_cum[i] = cc; cc += s_len[i]; }
+    int cc = 0, ss = 0;
+    for (int i = 0; i < nr; ++i) {
+      s_cum[i] = cc;
+      s_seg0[i] = ss;
+      cc += s_len[i];
+      if (s_len[i] > 0) ss += ((s_start[i] + s_len[i] - 1) >> p.page_shift) - (s_start[i] >> p.page_shift) + 1;
+    }
     s_cum[nr] = cc;
+    s_seg0[nr] = ss;
+    s_total_gone = 0;
   }
   __syncthreads();
-  const int count = s_cum[nr] < p.max_ctx_len ? s_cum[nr] : p.max_ctx_len;
+  const int all = s_cum[nr] < p.max_ctx_len ? s_cum[nr] : p.max_ctx_len;  // keys of the ranges, capped
+  const int n_seg = s_seg0[nr];
+  const bool compact = n_seg <= kMaxSegments;
+  const int page_mask = (1 << p.page_shift) - 1;
+  auto page_of = [&](int tok) {
+    int pi = tok >> p.page_shift;
+    pi = pi < 0 ? 0 : (pi >= p.bt_stride ? p.bt_stride - 1 : pi);
+    return p.block_table[(long)req * p.bt_stride + pi];
+  };
+  // ---- which pieces name no page, and how many keys are left out before each piece ----
+  bool any_gone = false;
+  if (compact) {
+    int mine[kMaxSegments / 256];
+#pragma unroll
+    for (int u = 0; u < kMaxSegments / 256; ++u) {
+      const int sg = tid * (kMaxSegments / 256) + u;   // a thread owns consecutive pieces: the prefix is in order
+      int gone = 0;
+      if (sg < n_seg) {
+        int rp = 0;
+        while (rp + 1 < nr && sg >= s_seg0[rp + 1]) ++rp;
+        const int pg = (s_start[rp] >> p.page_shift) + (sg - s_seg0[rp]);
+        const int t0 = pg << p.page_shift, t1 = t0 + page_mask + 1;
+        const int a = t0 > s_start[rp] ? t0 : s_start[rp];
+        const int b = t1 < s_start[rp] + s_len[rp] ? t1 : s_start[rp] + s_len[rp];
+        int v0 = s_cum[rp] + (a - s_start[rp]), v1 = s_cum[rp] + (b - s_start[rp]);
+        v0 = v0 < all ? v0 : all;
+        v1 = v1 < all ? v1 : all;
+        const int page = page_of(a);
+        if (v1 > v0 && (page < 0 || page >= p.n_pages)) gone = v1 - v0;
+      }
+      mine[u] = gone;
+    }
+    int sum = 0;
+#pragma unroll
+    for (int u = 0; u < kMaxSegments / 256; ++u) sum += mine[u];
+    any_gone = __syncthreads_or(sum != 0);
+    if (any_gone) {
+      int incl = sum;
+      const int lane = tid & 63, wv = tid >> 6;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int x = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += x;
+      }
+      if (lane == 63) s_wave[wv] = incl;
+      __syncthreads();
+      int before = incl - sum;
+      for (int w = 0; w < wv; ++w) before += s_wave[w];
+#pragma unroll
+      for (int u = 0; u < kMaxSegments / 256; ++u) {
+        const int sg = tid * (kMaxSegments / 256) + u;
+        if (sg < kMaxSegments) s_gone[sg] = before;
+        before += mine[u];
+      }
+      if (tid == 255) s_total_gone = before;
+      __syncthreads();
+    }
+  }
+  const int count = all - (any_gone ? s_total_gone : 0);
   int* row = table + (long)req * p.slot_stride;
   if (blockIdx.x == 0 && tid == 0) row[p.slot_stride - 1] = count;
   const int padded = (count + kKT - 1) / kKT * kKT;
-  const int v = blockIdx.x * 256 + tid;
-  if (v >= padded) return;
-  const int vv = v < count ? v : (v / kKT) * kKT;
+  const int v = blockIdx.x * 256 + tid;   // a key of the ranges (before anything is left out)
+  if (v >= all) return;
   int rp = 0;
-  while (rp + 1 < nr && vv >= s_cum[rp + 1]) ++rp;
-  const int tok = s_start[rp] + (vv - s_cum[rp]);
-  int pi = tok >> p.page_shift;
-  pi = pi < 0 ? 0 : (pi >= p.bt_stride ? p.bt_stride - 1 : pi);
-  int page = p.block_table[(long)req * p.bt_stride + pi];
-  page = page < 0 ? 0 : (page >= p.n_pages ? p.n_pages - 1 : page);
-  row[v] = (page << p.page_shift) + (tok & ((1 << p.page_shift) - 1));
+  while (rp + 1 < nr && v >= s_cum[rp + 1]) ++rp;
+  const int tok = s_start[rp] + (v - s_cum[rp]);
+  int page = page_of(tok);
+  int at = v;
+  if (any_gone) {
+    if (page < 0 || page >= p.n_pages) return;     // left out
+    const int sg = s_seg0[rp] + (tok >> p.page_shift) - (s_start[rp] >> p.page_shift);
+    at = v - s_gone[sg];
+  } else {
+    page = page < 0 ? 0 : (page >= p.n_pages ? p.n_pages - 1 : page);
+  }
+  const int slot = (page << p.page_shift) + (tok & page_mask);
+  row[at] = slot;
+  if (at == count - 1)
+    for (int o = count; o < padded; ++o) row[o] = slot;   // the ragged end of the last tile: a valid slot, masked
 }
 
 // Reduce the partial results of the columns that were cut into several pieces: one wave per

@@ -112,6 +112,51 @@ def test_shared_slot_table_matches_per_call_table(dev):
         assert t[r, :len(toks)].tolist() == want
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_page_table_entries_that_name_no_page_are_left_out(dev, fp8):
+    """The reference skips page-table entries of -1 (kv_cache_kernels.py:208).  Entries outside [0, n_pages) inside
+    the visible ranges -- a whole chunk's pages, the page in the middle of a range, the page a range ends in --
+    contribute no keys: the output equals the oracle's over the remaining keys, the slot table lists only those,
+    and a request whose visible pages are all gone attends to its active block alone."""
+    ops = _ops()
+    case = configs.chunked_prefix_case(23, n_req=4, n_chunks=6, chunk_tokens=300, topk=3, q_len=48,
+                                       shared_prefix=False, fp8=fp8)
+    n_pages = case.k_cache.shape[0]
+    bt = case.block_table.clone()
+    r0, r1, r3 = case.ranges[0], case.ranges[1], case.ranges[3]
+    bt[0, r0[0][0] // 256] = -1                                   # the page the first range starts in
+    bt[0, (r0[1][0] + 150) // 256] = n_pages + 5                  # a page in the middle of the second range
+    bt[1, (r1[2][0] + r1[2][1] - 1) // 256] = -1                  # the page the last range ends in
+    for start, length in r3:                                      # request 3: every visible page
+        bt[3, start // 256:(start + length - 1) // 256 + 1] = -1
+    case.block_table = bt
+    ref = oracle_case(case)
+    for kw in (dict(), dict(num_splits=3), dict(rows_per_group=256) if not fp8 else dict(rows_per_group=64)):
+        check(run_case(case, dev, **kw), ref, what=f"{kw}")
+    # request 3 sees its active block only
+    d = lambda t: None if t is None else t.to(dev)
+    a, b = int(case.q_start_loc[3]), int(case.q_start_loc[4])
+    alone = ref_ops.sparse_decode_attention(case.q[a:b], case.k_new[a:b], case.v_new[a:b], None, None, None,
+                                            [0, b - a], None)
+    assert_attn_close(run_case(case, dev)[a:b], alone, "request without a page")
+    # the table: the slots of the keys that remain, in order, then their number
+    rp, rs, rl, mr = case.range_tensors()
+    table = ops.new_slot_table(4, case.max_ctx, dev)
+    prep = ops.PreparedAttention(d(case.q), d(case.k_new), d(case.v_new), d(case.k_cache), d(case.v_cache), d(bt),
+                                 d(case.q_start_loc), max_q_len=case.max_q, max_ctx_len=case.max_ctx,
+                                 ranges=(d(rp), d(rs), d(rl), mr), slot_table=table, k_scale=d(case.k_scale),
+                                 v_scale=d(case.v_scale))
+    prep.build_slot_table()
+    torch.cuda.synchronize()
+    t = table.cpu()
+    for r, rr in enumerate(case.ranges):
+        toks = [s + i for s, l in rr for i in range(l)]
+        want = [int(bt[r, tk // 256]) * 256 + tk % 256 for tk in toks if 0 <= int(bt[r, tk // 256]) < n_pages]
+        assert int(t[r, -1]) == len(want) and t[r, :len(want)].tolist() == want
+        pad = (len(want) + 63) // 64 * 64
+        assert all(0 <= x < n_pages * 256 for x in t[r, len(want):pad].tolist())
+
+
 @pytest.mark.parametrize("rows", [0, 160, 256])
 def test_config3_shape_small_batch(dev, rows):
     case = configs.config3_small(seed=3, n_req=2)
