@@ -1143,31 +1143,30 @@ __global__ __launch_bounds__(256) void attn_slot_table_kernel(const AttnKParams 
   // ---- which pieces name no page, and how many keys are left out before each piece ----
   bool any_gone = false;
   if (compact) {
-    int mine[kMaxSegments / 256];
-#pragma unroll
-    for (int u = 0; u < kMaxSegments / 256; ++u) {
-      const int sg = tid * (kMaxSegments / 256) + u;   // a thread owns consecutive pieces: the prefix is in order
-      int gone = 0;
-      if (sg < n_seg) {
-        int rp = 0;
-        while (rp + 1 < nr && sg >= s_seg0[rp + 1]) ++rp;
-        const int pg = (s_start[rp] >> p.page_shift) + (sg - s_seg0[rp]);
-        const int t0 = pg << p.page_shift, t1 = t0 + page_mask + 1;
-        const int a = t0 > s_start[rp] ? t0 : s_start[rp];
-        const int b = t1 < s_start[rp] + s_len[rp] ? t1 : s_start[rp] + s_len[rp];
-        int v0 = s_cum[rp] + (a - s_start[rp]), v1 = s_cum[rp] + (b - s_start[rp]);
-        v0 = v0 < all ? v0 : all;
-        v1 = v1 < all ? v1 : all;
-        const int page = page_of(a);
-        if (v1 > v0 && (page < 0 || page >= p.n_pages)) gone = v1 - v0;
-      }
-      mine[u] = gone;
+    bool mine_gone = false;
+    for (int sg = tid; sg < n_seg; sg += 256) {
+      int rp = 0;
+      while (rp + 1 < nr && sg >= s_seg0[rp + 1]) ++rp;
+      const int pg = (s_start[rp] >> p.page_shift) + (sg - s_seg0[rp]);
+      const int t0 = pg << p.page_shift, t1 = t0 + page_mask + 1;
+      const int a = t0 > s_start[rp] ? t0 : s_start[rp];
+      const int b = t1 < s_start[rp] + s_len[rp] ? t1 : s_start[rp] + s_len[rp];
+      int v0 = s_cum[rp] + (a - s_start[rp]), v1 = s_cum[rp] + (b - s_start[rp]);
+      v0 = v0 < all ? v0 : all;
+      v1 = v1 < all ? v1 : all;
+      const int page = page_of(a);
+      const int gone = (v1 > v0 && (page < 0 || page >= p.n_pages)) ? v1 - v0 : 0;
+      s_gone[sg] = gone;
+      mine_gone |= gone != 0;
     }
-    int sum = 0;
-#pragma unroll
-    for (int u = 0; u < kMaxSegments / 256; ++u) sum += mine[u];
-    any_gone = __syncthreads_or(sum != 0);
+    any_gone = __syncthreads_or(mine_gone);
     if (any_gone) {
+      // exclusive prefix over the pieces, in place: a thread owns `per` consecutive pieces
+      const int per = (n_seg + 255) / 256;
+      const int s0 = tid * per < n_seg ? tid * per : n_seg;
+      const int s1 = s0 + per < n_seg ? s0 + per : n_seg;
+      int sum = 0;
+      for (int sg = s0; sg < s1; ++sg) sum += s_gone[sg];
       int incl = sum;
       const int lane = tid & 63, wv = tid >> 6;
 #pragma unroll
@@ -1179,11 +1178,10 @@ __global__ __launch_bounds__(256) void attn_slot_table_kernel(const AttnKParams 
       __syncthreads();
       int before = incl - sum;
       for (int w = 0; w < wv; ++w) before += s_wave[w];
-#pragma unroll
-      for (int u = 0; u < kMaxSegments / 256; ++u) {
-        const int sg = tid * (kMaxSegments / 256) + u;
-        if (sg < kMaxSegments) s_gone[sg] = before;
-        before += mine[u];
+      for (int sg = s0; sg < s1; ++sg) {
+        const int g = s_gone[sg];
+        s_gone[sg] = before;
+        before += g;
       }
       if (tid == 255) s_total_gone = before;
       __syncthreads();
