@@ -208,6 +208,9 @@ def x_decode_32_rows(torch, ops, dev, gd):
             "plan": p32[0].attn.describe_plan()}
 
 
+PREFILL_NUM_SPLITS = 0   # --num-splits with --only prefill: 1 = one workgroup per column (attn_fwd_kernel)
+
+
 def _prefill_inputs(torch, ops, dev, gd):
     """configs[3]: 32 chunks x (1 BOS + 1024) tokens, Q/K/V drawn N(0,1), a seeded page table."""
     L, NC = 1025, 32
@@ -229,11 +232,26 @@ def x_prefill(torch, ops, dev, gd):
     a prefill is 28 of these)."""
     L, NC, q, k, v, kc, vc, slots, cu = _prefill_inputs(torch, ops, dev, gd)
     o = torch.empty_like(q)
+    ns = PREFILL_NUM_SPLITS
     us = _time_us(torch, lambda: ops.chunk_prefill_attention(q, k, v, cu, max_seqlen=L, causal=True, k_cache=kc,
-                                                             v_cache=vc, slot_mapping=slots, out=o), 5, 1)
+                                                             v_cache=vc, slot_mapping=slots, out=o, num_splits=ns), 5, 1)
     fl = 2.0 * NC * L * L * D * HQ
     return {"us_per_layer": us, "bf16_TFLOPs": fl / us / 1e6, "mfma_frac": fl / us / 1e6 / PEAK_BF16_TFLOPS,
-            "us_per_prefill_28_layers": us * 28, "inputs": "N(0,1)"}
+            "us_per_prefill_28_layers": us * 28, "inputs": "N(0,1)",
+            "plan": ops.describe_prefill_plan(NC, HQ, HKV, L, NC * L, causal=True, num_splits=ns)}
+
+
+def x_prefill_full(torch, ops, dev, gd):
+    """The rows of configs[3] with every key of their chunk visible and no store (17 tiles per column, no mask):
+    the rate of the prefill kernel's tile loop without the short columns of the causal case."""
+    L, NC, q, k, v, kc, vc, slots, cu = _prefill_inputs(torch, ops, dev, gd)
+    o = torch.empty_like(q)
+    ns = PREFILL_NUM_SPLITS
+    us = _time_us(torch, lambda: ops.chunk_prefill_attention(q, k, v, cu, max_seqlen=L, causal=False, out=o,
+                                                             num_splits=ns), 5, 1)
+    fl = 4.0 * NC * L * L * D * HQ
+    return {"us_per_layer": us, "bf16_TFLOPs": fl / us / 1e6, "mfma_frac": fl / us / 1e6 / PEAK_BF16_TFLOPS,
+            "plan": ops.describe_prefill_plan(NC, HQ, HKV, L, NC * L, causal=False, num_splits=ns)}
 
 
 def x_rope_qk_store(torch, ops, dev, gd):
@@ -379,6 +397,7 @@ def x_fp8(torch, ops, dev, gd):
 EXTRAS = collections.OrderedDict([
     ("decode_32_rows", ("decode32", x_decode_32_rows)),
     ("prefill_32x1025_causal_layer", ("prefill", x_prefill)),
+    ("prefill_32x1025_full_mask_layer_no_store", ("prefillfull", x_prefill_full)),
     ("rope_qk_store_32x1025_layer", ("rope", x_rope_qk_store)),
     ("score_32x4x152064_top4", ("score", x_score)),
     ("evict_8x28x64x1025_keep256", ("evict", x_evict)),
@@ -445,6 +464,8 @@ def main():
         del src, dst
 
     if args.only:
+        global PREFILL_NUM_SPLITS
+        PREFILL_NUM_SPLITS = args.num_splits
         only = set(args.only.split(","))
         unknown = only - {v[0] for v in EXTRAS.values()}
         if unknown:
