@@ -360,7 +360,10 @@ int pdllm_kv_copy_pages(const void* src_cache, void* dst_cache, const int32_t* s
  * vocabularies up to 152064).  Everything that compares the confidence with a threshold (pdllm_threshold_unmask,
  * pdllm_denoise_unmask*) therefore decides exactly as the reference whenever the reference's confidence is
  * further than 5e-5 from the threshold; inside that band either decision can come out.  The most confident
- * position of a block is always transferred, so a block never stalls on such a tie. */
+ * position of a block is always transferred, so a block never stalls on such a tie.
+ * Limit: n_seqs * block_len <= 65535 rows per call (one grid dimension of the scan); more returns
+ * PDLLM_ERR_UNSUPPORTED, here and in pdllm_denoise_unmask and pdllm_denoise_unmask_static (where an input
+ * of that size also exceeds the static scratch area, whichever check comes first). */
 int pdllm_conf_argmax(const void* logits, int64_t logits_stride, const void* last_logit,
                       int64_t last_logit_stride, int64_t n_seqs, int64_t block_len, int64_t vocab,
                       int32_t shift, void* workspace, int64_t workspace_bytes, float* conf_out,

@@ -1390,7 +1390,10 @@ static int validate_desc(const pdllm_attn_desc* d, bool prefill) {
     if (d->cache_head_stride != kD || d->cache_token_stride != hk ||
         d->cache_page_stride != hk * d->page_size)
       return PDLLM_ERR_STRIDE;
-    if (((uintptr_t)d->k_cache | (uintptr_t)d->v_cache | (uintptr_t)d->active_slot_mapping) % 4) return PDLLM_ERR_STRIDE;
+    // the store kernels write 16 bytes per lane (8 per lane of fp8 bytes), with or without a visible prefix
+    const uintptr_t salign = d->kv_dtype == PDLLM_KV_FP8_E4M3 ? 8 : 16;
+    if (((uintptr_t)d->k_cache | (uintptr_t)d->v_cache) % salign) return PDLLM_ERR_STRIDE;
+    if ((uintptr_t)d->active_slot_mapping % 4) return PDLLM_ERR_STRIDE;
   }
   if (has_cache && d->slot_table != nullptr) {
     if (d->slot_table_stride < slot_table_stride_for(d) || ((uintptr_t)d->slot_table % 4)) return PDLLM_ERR_STRIDE;

@@ -89,6 +89,34 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert ada(p, 128, p, 128, None, 0, 0, None, o, 128, p, 0, 4, 0, 128, 4, 3, 3, 0, 0, 1.0, 1.0, 0, None) == 0    # nothing to do
 
 
+def test_store_only_descriptor_needs_aligned_cache():
+    """A decode call without a visible prefix that still stores its active rows (active_slot_mapping set,
+    max_ctx_len 0) writes 16 bytes per lane (8 of fp8 bytes): a cache base that is not aligned to that is refused on
+    the host, as it is when a prefix is read."""
+    from prefilling_dllm_amd import _lib
+    lib = _lib.lib
+    buf = (ctypes.c_char * 256)()
+    p = (ctypes.addressof(buf) + 63) & ~63
+    d = _lib.AttnDesc()
+    d.q = d.k_new = d.v_new = d.out = d.q_start_loc = d.active_slot_mapping = p
+    d.head_dim, d.num_q_heads, d.num_kv_heads = 128, 28, 4
+    d.q_stride = d.o_stride = 28 * 128
+    d.kn_stride = d.vn_stride = 4 * 128
+    d.n_tokens, d.n_req, d.max_q_len, d.max_ctx_len = 32, 1, 32, 0
+    d.mask_mode, d.sm_scale = _lib.MASK_FULL, 0.088
+    d.kv_dtype, d.page_size, d.n_pages = _lib.KV_BF16, 256, 2
+    d.cache_head_stride, d.cache_token_stride, d.cache_page_stride = 128, 512, 512 * 256
+    d.k_cache = d.v_cache = p
+    assert lib.pdllm_attn_workspace_bytes(ctypes.byref(d)) >= 0
+    d.k_cache = p + 8
+    assert lib.pdllm_attn_workspace_bytes(ctypes.byref(d)) == -3
+    d.kv_dtype = _lib.KV_FP8_E4M3                      # fp8 rows: 8-byte stores
+    d.k_scale = d.v_scale = p
+    assert lib.pdllm_attn_workspace_bytes(ctypes.byref(d)) >= 0
+    d.k_cache = p + 4
+    assert lib.pdllm_attn_workspace_bytes(ctypes.byref(d)) == -3
+
+
 def test_attention_plan_is_host_only():
     from prefilling_dllm_amd import ops
     rows, splits = ops.attention_plan(8, 28, 4, max_q_len=160, max_ctx_len=4096)
@@ -221,6 +249,85 @@ def test_page_pool_semantics():
     assert a.allocate_pages(4) == [3, 0, 1, 2] and a.num_free_pages == 0 and list(a.free_pages) == []
     a.release_pages([1])
     assert list(a.free_pages) == [1]
+
+
+def test_page_pool_edge_cases():
+    """Nothing asked for is nothing done (the reference returns [] for n <= 0, fastdllm_engine.py:112-119), and a
+    release that must be refused leaves the pool as it was."""
+    from prefilling_dllm_amd.page_pool import PagePool
+    a = PagePool(4, 256)
+    assert a.allocate_pages(0) == [] and a.allocate_pages(-2) == [] and a.num_free_pages == 4
+    assert list(a.free_pages) == [0, 1, 2, 3]
+    p = a.allocate_pages(3)                                       # [0, 1, 2], one holder each
+    a.ref_pages([1])
+    before = (a.num_free_pages, list(a.free_pages), [a.page_ref_count[i] for i in range(4)])
+    with pytest.raises(RuntimeError, match="released more often"):
+        a.release_pages([0, 1, 1, 1])                             # page 1 has two holders, three are dropped
+    with pytest.raises(RuntimeError, match="released more often"):
+        a.release_pages([2, 2])
+    with pytest.raises(RuntimeError, match="not all pages of this pool"):
+        a.release_pages([0, 7])
+    assert (a.num_free_pages, list(a.free_pages), [a.page_ref_count[i] for i in range(4)]) == before
+    a.release_pages([])                                           # nothing listed
+    a.release_pages([1, 1, 0])                                    # a page listed twice drops two holders
+    assert list(a.free_pages) == [3, 1, 0] and p == [0, 1, 2]
+
+
+def test_normalize_per_head_keep_indices_contract():
+    """_normalize_per_head_keep_indices (fastdllm_engine.py:560-605): one [heads, n] index tensor per layer, one
+    common n, entries inside the prompt; the error names the first offending layer."""
+    import torch
+    from prefilling_dllm_amd.engine_ops import normalize_per_head_keep_indices as norm
+    kw = dict(num_layers=3, num_heads=2, full_prompt_len=10, device="cpu")
+    good = [[[0, 3, 9], [1, 2, 3]], torch.tensor([[4, 5, 6], [7, 8, 9]], dtype=torch.int32), [[0, 1, 2], [0, 1, 2]]]
+    out, n = norm(good, **kw)
+    assert n == 3 and len(out) == 3 and all(t.dtype == torch.int64 and t.is_contiguous() for t in out)
+    assert out[1].tolist() == [[4, 5, 6], [7, 8, 9]]
+    assert norm([], num_layers=0, num_heads=2, full_prompt_len=10, device="cpu") == ([], 0)
+    empty, n0 = norm([torch.zeros(2, 0, dtype=torch.long)] * 3, **kw)
+    assert n0 == 0 and len(empty) == 3
+    with pytest.raises(ValueError, match="2 layers"):
+        norm(good[:2], **kw)
+    with pytest.raises(ValueError, match="layer 1"):
+        norm([good[0], [[1, 2, 3]], good[2]], **kw)                      # one head instead of two
+    with pytest.raises(ValueError, match="layer 2"):
+        norm([good[0], good[1], [[0, 1], [0, 1]]], **kw)                 # another active length
+    with pytest.raises(ValueError, match="layer 0"):
+        norm([[0, 1, 2], good[1], good[2]], **kw)                        # not two-dimensional
+    with pytest.raises(ValueError, match="layer 1.*outside the prompt of 10"):
+        norm([good[0], [[4, 5, 10], [7, 8, 9]], [[0, 1, -1], [0, 1, 2]]], **kw)
+    with pytest.raises(ValueError, match="layer 2.*outside"):
+        norm([good[0], good[1], [[0, 1, -1], [0, 1, 2]]], **kw)
+
+
+def test_active_block_mask_from_per_sequence_masks():
+    """Per-sequence masks [h, ctx + h] (engine/sequence.py:489-493) -> the block-diagonal [Nq, Nq] mask over the
+    active keys that utils/context.py:73-98 lays out, None when nothing is hidden; a hidden context key is refused."""
+    import torch
+    from prefilling_dllm_amd.context import active_block_mask, ContextForDiffusionLM
+    from types import SimpleNamespace
+    assert active_block_mask([]) is None
+    full = [torch.ones(1, 1, 3, 8, dtype=torch.bool), torch.ones(2, 2, dtype=torch.bool)]
+    assert active_block_mask(full) is None
+    a = torch.ones(3, 8, dtype=torch.bool)
+    a[0, 6:] = False                                   # row 0 does not see active keys 1, 2
+    b = torch.tensor([[1, 0], [1, 1]], dtype=torch.bool)
+    got = active_block_mask([a.view(1, 1, 3, 8), b])
+    want = torch.zeros(5, 5, dtype=torch.bool)
+    want[:3, :3] = a[:, 5:]
+    want[3:, 3:] = b
+    assert torch.equal(got, want)
+    hidden_ctx = torch.ones(3, 8, dtype=torch.bool)
+    hidden_ctx[1, 2] = False
+    with pytest.raises(ValueError, match="hides cached context keys"):
+        active_block_mask([hidden_ctx])
+    with pytest.raises(ValueError, match="only 2 key columns"):
+        active_block_mask([torch.ones(3, 2, dtype=torch.bool)])
+    # the context assembles it from its sequences, as the reference's __post_init__ does
+    ctx = ContextForDiffusionLM(seqs=[SimpleNamespace(current_block_mask=a), SimpleNamespace(current_block_mask=b)])
+    assert ctx.mask_kind == "dense" and torch.equal(ctx.block_mask, want)
+    ctx = ContextForDiffusionLM(seqs=[SimpleNamespace(current_block_mask=m) for m in full])
+    assert ctx.block_mask is None and ctx.mask_kind == "full"
 
 
 def test_record_helpers_take_any_allocator():

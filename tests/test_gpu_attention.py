@@ -513,6 +513,55 @@ def test_attention_layer_interface(dev):
     assert torch.equal(kc[3, :block], k2.view(-1, Hkv, d))
 
 
+def test_store_before_attention_for_callers_that_rewrite_visible_rows(dev, monkeypatch):
+    """A decode step normally stores its active rows inside the attention call, after the kernel has read the cache;
+    that equals the reference's store-then-attend order (attention_v4.py:328-331) only while no active slot is a
+    visible prefix slot.  A caller that rewrites visible context rows sets `store_before_attention`: the output is then
+    the oracle's over the cache *after* the store.  Without the flag the debug check names the violation."""
+    from prefilling_dllm_amd.attention import Attention
+    from prefilling_dllm_amd.context import set_context_diffusion_lm, reset_context_diffusion_lm
+    gen = torch.Generator().manual_seed(53)
+    Hq, Hkv, d, P = 28, 4, 128, 256
+    ctx, block = 300, 32
+    layer = Attention(Hq, d, d ** -0.5, Hkv, "diffusion_lm")
+    kc0 = (torch.randn(4, P, Hkv, d, generator=gen) / 3).to(torch.bfloat16)
+    vc0 = (torch.randn(4, P, Hkv, d, generator=gen) / 3).to(torch.bfloat16)
+    bt = torch.tensor([[2, 0]], dtype=torch.int32)
+    mk = lambda n, h: (torch.randn(n, h * d, generator=gen) / 3).to(torch.bfloat16)
+    q, k, v = mk(block, Hq), mk(block, Hkv), (mk(block, Hkv).float() + 2.0).to(torch.bfloat16)
+    # the block overwrites context tokens 100 .. 131 (page 2 of the cache), which every row can see
+    slots = (2 * P + 100 + torch.arange(block)).to(torch.int32)
+    cu = torch.tensor([0, block], dtype=torch.int32, device=dev)
+    common = dict(cu_seqlens_q=cu, max_seqlen_q=block, max_seqlen_k=ctx + block, slot_mapping=slots.to(dev),
+                  context_lens=torch.tensor([ctx], dtype=torch.int32, device=dev), block_tables=bt.to(dev),
+                  mask_kind="full")
+    kc_ref, vc_ref = kc0.clone(), vc0.clone()
+    ref_ops.store_kvcache(k.view(-1, Hkv, d), v.view(-1, Hkv, d), kc_ref, vc_ref, slots)
+    ref = ref_ops.sparse_decode_attention(q.view(-1, Hq, d), k.view(-1, Hkv, d), v.view(-1, Hkv, d), kc_ref, vc_ref,
+                                          bt, [0, block], [[(0, ctx)]])
+    stale = ref_ops.sparse_decode_attention(q.view(-1, Hq, d), k.view(-1, Hkv, d), v.view(-1, Hkv, d), kc0, vc0,
+                                            bt, [0, block], [[(0, ctx)]])
+    assert (ref - stale).abs().max() > 0.05            # the order matters for this input
+    layer.k_cache, layer.v_cache = kc0.to(dev), vc0.to(dev)
+    set_context_diffusion_lm(False, store_before_attention=True, **common)
+    try:
+        o = layer(q.to(dev), k.to(dev), v.to(dev))
+    finally:
+        reset_context_diffusion_lm()
+    check(o.view(-1, Hq, d).float().cpu(), ref, tol=3e-2)
+    assert torch.equal(layer.k_cache.cpu(), kc_ref) and torch.equal(layer.v_cache.cpu(), vc_ref)
+    # without the flag, under the debug check: refused before anything is launched or stored
+    layer.k_cache, layer.v_cache = kc0.to(dev), vc0.to(dev)
+    monkeypatch.setenv("PDLLM_DEBUG_CHECKS", "1")
+    set_context_diffusion_lm(False, **common)
+    try:
+        with pytest.raises(RuntimeError, match="store_before_attention"):
+            layer(q.to(dev), k.to(dev), v.to(dev))
+    finally:
+        reset_context_diffusion_lm()
+    assert torch.equal(layer.k_cache.cpu(), kc0)
+
+
 def test_reference_form_decode_masks_with_context_columns(dev):
     """The reference hands the layer per-sequence masks [Sq, ctx + Sq] (fastdllm_engine.py:496-507: all ones, with
     the keys behind `valid_tokens` hidden from the first `valid_tokens` rows) through `seqs`, or the block-diagonal
