@@ -374,6 +374,53 @@ def test_chunk_prefill_stream_kernel(dev, lens, heads, causal):
         check(a.float().cpu(), ref, tol=3e-2)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_chunk_prefill_stream_kernel_random_batches(dev, seed):
+    """Seeded random batches for the stream kernel: ragged chunk lengths with empty chunks, one-token chunks and
+    lengths on both sides of a tile boundary, 1 to 16 query heads per KV head, logits that grow along the keys (the
+    running maximum moves in late tiles: accumulators that carry weight are rescaled), causal and full masks.  The
+    result must equal one workgroup per column up to the rounding of the output: the decision to rescale is taken
+    per wave, and in a wave that also holds rows past the end of its chunk it depends on what those lanes hold, which
+    the two kernels fill differently -- such rows may differ by one bf16 step, every other row is equal bit for bit."""
+    ops = _ops()
+    rng = torch.Generator().manual_seed(1000 + seed)
+    Hq, Hkv = [(28, 4), (8, 8), (16, 8), (32, 8), (16, 2), (32, 2)][seed]
+    G = Hq // Hkv
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=rng))
+    special = [0, 1, 63, 64, 65, 127, 128, 129, 1024, 1025]
+    # enough rows per chunk for 16 columns of 128 rows (R >= team) at the largest chunk, enough units for the teams
+    lmax = max(pick(1100, 1600), (16 * 128 + G - 1) // G + 1)
+    n_chunks = max(8, 2 * (512 // 16) // Hkv + pick(0, 3))
+    lens = [lmax] + [special[pick(0, len(special) - 1)] if pick(0, 3) == 0 else pick(1, lmax) for _ in range(n_chunks - 1)]
+    causal = seed % 2 == 0
+    n, dd = sum(lens), 128
+    q = torch.randn(n, Hq, dd, generator=rng).to(torch.bfloat16)
+    k = torch.randn(n, Hkv, dd, generator=rng)
+    # keys late in a chunk carry larger logits: ramp their norm along the chunk
+    pos = torch.cat([torch.arange(l) for l in lens]).float()
+    k = (k * (1.0 + pos[:, None, None] / 400.0)).to(torch.bfloat16)
+    v = torch.randn(n, Hkv, dd, generator=rng).to(torch.bfloat16)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    plan = ops.describe_prefill_plan(len(lens), Hq, Hkv, max(lens), n, causal)
+    assert "attn_prefill_stream_kernel" in plan, (plan, lens, Hq, Hkv)
+    a = ops.chunk_prefill_attention(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), max_seqlen=max(lens), causal=causal)
+    b = ops.chunk_prefill_attention(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), max_seqlen=max(lens), causal=causal,
+                                    num_splits=1)
+    torch.cuda.synchronize()
+    af, bf = a.float().cpu(), b.float().cpu()
+    assert torch.isfinite(af).all()
+    differ = (af != bf).flatten(1).any(dim=1)
+    assert int(differ.sum()) <= len(lens) * max(1, 32 // G + 1), (seed, int(differ.sum()))   # last row blocks of chunks at most
+    row_scale = bf.abs().amax(dim=2, keepdim=True).clamp_min(2.0 ** -7)          # one bf16 step of the row's largest
+    assert ((af - bf).abs() <= 2.0 ** -7 * row_scale).all(), (seed, (af - bf).abs().max())
+    # one mid-sized chunk against the oracle
+    c = max(range(len(lens)), key=lambda i: lens[i] if lens[i] <= 700 else 0)
+    if lens[c] > 0:
+        lo, hi = int(cu[c]), int(cu[c + 1])
+        ref = ref_ops.chunk_prefill_attention(q[lo:hi], k[lo:hi], v[lo:hi], [0, hi - lo], causal=causal)
+        check(a[lo:hi].float().cpu(), ref, tol=3e-2)
+
+
 def test_permuting_pages_leaves_output_unchanged(dev):
     """Size-independent property: the physical page order is irrelevant (same logical tokens)."""
     case = configs.chunked_prefix_case(13, n_req=1, n_chunks=4, chunk_tokens=512, topk=4, q_len=32)
