@@ -45,6 +45,7 @@ struct PrefillParams {
   const int* q_start_loc;
   long q_stride, o_stride;  // elements
   unsigned kv_row_bytes;    // token pitch of k and of v (equal), bytes
+  unsigned out_bytes;       // bytes from out to the end of its last row
   long n_tokens;
   int n_req, Hq, Hkv, G;
   int causal;
@@ -178,6 +179,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_stream_kernel(const Prefi
   unsigned wave_lds = lds_base + wave * 1024;
   const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(p.k), 0, 0xffffffff, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(p.v), 0, 0xffffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(p.q), 0, 0xffffffff, 0x00020000);
+  // the output's size in bytes bounds its stores: offsets of rows that do not exist lie behind it
+  const __amdgpu_buffer_rsrc_t o_rs = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, p.out_bytes, 0x00020000);
   // copy group i of tile `tile` of column pc into LDS offset dst_off of this wave's part
   // (whole_tag: the tile is known to be a whole tile of the column)
   auto copy_group = [&](const __amdgpu_buffer_rsrc_t& rs, const Piece& pc, int tile, int i, unsigned dst_off,
@@ -237,12 +241,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_stream_kernel(const Prefi
     const int rr = r < pc.Sq * G ? r : pc.row0;
     const int tq = rr / G;
     const int g = rr - tq * G;
-    return p.q + (long)(pc.q0 + tq) * p.q_stride + (long)(pc.kvh * G + g) * kD + 8 * (lane_e >> 5);
+    // byte offset behind p.q (the launch is made only when Q and the output lie below 4 GiB: a buffer load with a
+    // 32-bit offset costs the issuing wave a fraction of a load with a 64-bit address per lane)
+    return 2u * ((unsigned)(pc.q0 + tq) * (unsigned)p.q_stride + (unsigned)((pc.kvh * G + g) * kD + 8 * (lane_e >> 5)));
   };
   auto load_q = [&](const Piece& pc) __attribute__((always_inline)) {
-    const __bf16* qp = q_address(pc);
+    const unsigned qo = q_address(pc);
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) QA[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+    for (int ks = 0; ks < 8; ++ks)
+      QA[ks] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(q_rs, (int)qo + 32 * ks, 0, 0));
   };
 
   f32x16 OA[4];
@@ -264,13 +271,14 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_stream_kernel(const Prefi
     const float lsum = half_swap_sum(lA);
     const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
     const int r = pc.row0 + 32 * wave + l32e;
-    unsigned long rowptr = 0;  // global address of this lane's row, 0 = no such row
+    // byte offset of this lane's row behind p.out; a row that does not exist gets an offset past the buffer's
+    // size, and the hardware drops a buffer store that lies out of range
+    unsigned rowoff = 0xfffff000u;
     if (r < pc.Sq * G) {
       const int srow = row_token(pc, lane_e);
       const int g = r - srow * G;
-      rowptr = (unsigned long)(p.out + (long)(pc.q0 + srow) * p.o_stride + (long)(pc.kvh * G + g) * kD);
+      rowoff = 2u * ((unsigned)(pc.q0 + srow) * (unsigned)p.o_stride + (unsigned)((pc.kvh * G + g) * kD));
     }
-    const int ptr_lo = (int)(unsigned)rowptr, ptr_hi = (int)(unsigned)(rowptr >> 32);
     char* strip = lds + par * kBufBytes + kTileBytes + wave * 1024;
     char* wrow = strip + (l32e >> 3) * 4096 + (l32e & 7) * 128 + 8 * he;
     const int wsw = (l32e >> 1) & 7;
@@ -290,9 +298,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_stream_kernel(const Prefi
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const int rr = 8 * k + (lane_e >> 3);
-        const unsigned long dst = ((unsigned long)(unsigned)__shfl(ptr_hi, rr, 64) << 32) | (unsigned)__shfl(ptr_lo, rr, 64);
-        const uint4 x = *reinterpret_cast<const uint4*>(strip + k * 4096 + (rr & 7) * 128 + ((j ^ ((rr >> 1) & 7)) << 4));
-        if (dst != 0) *reinterpret_cast<uint4*>(dst + 2 * (64 * hf + 8 * j)) = x;
+        const unsigned dst = (unsigned)__shfl((int)rowoff, rr, 64);
+        typedef unsigned u32x4s __attribute__((ext_vector_type(4)));
+        const u32x4s x = *reinterpret_cast<const u32x4s*>(strip + k * 4096 + (rr & 7) * 128 + ((j ^ ((rr >> 1) & 7)) << 4));
+        __builtin_amdgcn_raw_buffer_store_b128(x, o_rs, (int)(dst + 2u * (64 * hf + 8 * j)), 0, 0);
       }
     }
     MA = -INFINITY;
@@ -623,6 +632,8 @@ bool prefill_stream_plan(const pdllm_attn_desc* d, int cus, int* grid, int* team
   if (d->kn_stride != d->vn_stride) return false;
   const int64_t row_b = d->kn_stride * 2;
   if (d->n_tokens >= (1l << 24) || row_b >= (1l << 24) || d->n_tokens * row_b >= (1l << 32) - 4096) return false;
+  // Q and the output are addressed with 32-bit byte offsets as well
+  if (d->n_tokens * d->q_stride * 2 >= (1l << 32) - 8192 || d->n_tokens * d->o_stride * 2 >= (1l << 32) - 8192) return false;
   const int G = d->num_q_heads / d->num_kv_heads;
   const long R = ((long)d->max_q_len * G + 127) / 128;
   const long units = (long)d->n_req * d->num_kv_heads;
@@ -650,6 +661,7 @@ int launch_prefill_stream(const pdllm_attn_desc* d, int grid, int team, hipStrea
   p.q_stride = d->q_stride;
   p.o_stride = d->o_stride;
   p.kv_row_bytes = (unsigned)(d->kn_stride * 2);
+  p.out_bytes = (unsigned)(((d->n_tokens - 1) * d->o_stride + (int64_t)d->num_q_heads * kD) * 2);
   p.n_tokens = d->n_tokens;
   p.n_req = d->n_req;
   p.Hq = d->num_q_heads;
