@@ -58,8 +58,8 @@ def test_config4_full_prefill_layer(dev):
     out = ops.chunk_prefill_attention(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), max_seqlen=L, causal=True,
                                       k_cache=kc, v_cache=vc, slot_mapping=slots).float().cpu()
     assert torch.isfinite(out).all()
-    # block-diagonal == independent per-chunk causal attention (oracle on three of the 32 chunks)
-    for c in (0, 13, 31):
+    # block-diagonal == independent per-chunk causal attention (the oracle on every chunk)
+    for c in range(NC):
         sl = slice(c * L, (c + 1) * L)
         ref = ref_ops.chunk_prefill_attention(q[sl], k[sl], v[sl], torch.tensor([0, L]), causal=True)
         assert_attn_close(out[sl], ref, f"C4 chunk {c}")
@@ -106,8 +106,8 @@ def test_config5_full_fp8_decode_layer_and_unmask(dev):
     assert "kv=fp8 row_blocks=5 " in prep.describe_plan(), prep.describe_plan()
     out = prep.run().float().cpu()
     assert torch.isfinite(out).all()
-    # oracle on the first and last request (dequantised pages)
-    for r in (0, 3):
+    # the oracle on every request (dequantised pages)
+    for r in range(4):
         a, b = int(case.q_start_loc[r]), int(case.q_start_loc[r + 1])
         ref = ref_ops.sparse_decode_attention(case.q[a:b], case.k_new[a:b], case.v_new[a:b], case.k_cache_ref,
                                               case.v_cache_ref, case.block_table[r:r + 1], torch.tensor([0, b - a]),
