@@ -260,6 +260,18 @@ int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t n_heads, in
                        int64_t n_keys, int64_t heads_per_group, void* workspace,
                        int64_t workspace_bytes, float* scores_out, pdllm_stream_t stream);
 
+/* One eviction step from ready-made probabilities in one call: pdllm_evict_colsum followed by
+ * pdllm_topb_keep_bos on its scores (fastdllm_engine.py:1230-1322 summed over queries and heads, then :903-927),
+ * same scores and same indices bit for bit.  scores_out [n_chunks, n_groups, n_keys] fp32, indices_out
+ * [n_chunks * n_groups, keep] int64 ascending with keep = min(max(capacity, 1), n_keys).  With a workspace of
+ * pdllm_evict_colsum_workspace_bytes() bytes, few chunks and n_keys <= 2048 the step is two launches (per-head
+ * column sums; then the sum over the heads of a group and the selection, one workgroup per row); otherwise it is
+ * the launches of the two calls. */
+int pdllm_evict_keep_from_probs(const float* probs, int64_t n_chunks, int64_t n_heads, int64_t n_queries,
+                                int64_t n_keys, int64_t heads_per_group, int64_t capacity, int32_t keep_high,
+                                int32_t force_keep_first, void* workspace, int64_t workspace_bytes,
+                                float* scores_out, int64_t* indices_out, pdllm_stream_t stream);
+
 /* Replaces query_to_chunk_attention_scores (OPS/triton_eviction_scorer.py:114-210) and
  * the torch path of _engine_chunk_attention_head_scores (ENG:1279-1310): q [S, Hq, d],
  * k [S, Hkv, d] bf16 contiguous, S = prefix_len + chunk_len + query_len; for every

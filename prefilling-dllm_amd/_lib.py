@@ -73,6 +73,7 @@ SIGNATURES = {
     "pdllm_topk_lowest_index": (C.c_int, [vp, i64, i64, i64, i64, i32, vp, vp]),
     "pdllm_evict_colsum": (C.c_int, [vp, i64, i64, i64, i64, i64, vp, i64, vp, vp]),
     "pdllm_evict_colsum_workspace_bytes": (i64, [i64, i64, i64]),
+    "pdllm_evict_keep_from_probs": (C.c_int, [vp, i64, i64, i64, i64, i64, i64, i32, i32, vp, i64, vp, vp, vp]),
     "pdllm_kv_compact_per_head_workspace_bytes": (i64, [i64, i32, i32, i32]),
     "pdllm_kv_compact_per_head": (C.c_int, [vp, i64, i32, vp, i64, vp, i64, i64, i64, i32, i32, i32, i64, i32, vp, i64, vp]),
     "pdllm_evict_score_qk_workspace_bytes": (i64, [i64, i64, i64, i32, i32, i32]),

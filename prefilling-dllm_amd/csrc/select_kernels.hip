@@ -6,6 +6,7 @@
 // :1230-1322 + layers/attention/ops/triton_eviction_scorer.py:6-210 (eviction scores),
 // :1405-1433 (pooling and per-KV-head grouping) of the reference engine.
 
+#include <type_traits>
 #include "pdllm_common.h"
 
 namespace pdllm {
@@ -317,6 +318,126 @@ __global__ __launch_bounds__(256) void evict_groupsum_kernel(const float* __rest
   out[(chunk * n_groups + g) * n_keys + c] = acc;
 }
 
+
+// Sum over the heads of a group and the keep set of the row in one launch: evict_groupsum_kernel followed by
+// topk_radix_kernel<true> with position 0 forced first, for rows of at most 2048 keys.  One workgroup of 1024
+// threads per (chunk, group): thread t owns keys t and t + 1024, adds their per-head sums in head order (the same
+// additions as evict_groupsum_kernel: the scores it writes are the same bits), keeps the two 32-bit keys in
+// registers and finds the k-th best key by four 8-bit radix passes over a histogram in LDS.  A segment of 1024
+// consecutive keys is laid over the threads in index order, so the position of a kept key in the ascending output is a
+// count over wave ballots.
+constexpr int kSelThreads = 1024;
+__global__ __launch_bounds__(kSelThreads) void evict_groupsum_select_kernel(
+    const float* __restrict__ hsum, long n_heads, long hpg, long n_keys, long k, int descending, int force_first,
+    float* __restrict__ scores, long* __restrict__ out) {
+  __shared__ int hist[256];
+  __shared__ int scan_tot[4];
+  __shared__ uint32_t s_prefix;
+  __shared__ int s_need;
+  __shared__ int seg_lt[2][16], seg_eq[2][16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const long row = blockIdx.x;
+  const long n_groups = n_heads / hpg;
+  const long chunk = row / n_groups, g = row - chunk * n_groups;
+  uint32_t key[2];
+  bool valid[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const long c = tid + 1024L * u;
+    valid[u] = c < n_keys;
+    key[u] = 0xffffffffu;
+    if (valid[u]) {
+      const float* src = hsum + (chunk * n_heads + g * hpg) * n_keys + c;
+      float acc = 0.f;
+      long hh = 0;
+      // batches of 32, 28, 16, 8, 4, 2, 1 loads in flight (a group of 28 or 32 heads: one round trip), added in
+      // head order
+      auto batch = [&](auto n_tag) __attribute__((always_inline)) {
+        constexpr int N = decltype(n_tag)::value;
+        float v[N];
+#pragma unroll
+        for (int x = 0; x < N; ++x) v[x] = src[(hh + x) * n_keys];
+#pragma unroll
+        for (int x = 0; x < N; ++x) acc += v[x];
+        hh += N;
+      };
+      while (hh + 32 <= hpg) batch(std::integral_constant<int, 32>{});
+      if (hh + 28 <= hpg) batch(std::integral_constant<int, 28>{});
+      if (hh + 16 <= hpg) batch(std::integral_constant<int, 16>{});
+      if (hh + 8 <= hpg) batch(std::integral_constant<int, 8>{});
+      if (hh + 4 <= hpg) batch(std::integral_constant<int, 4>{});
+      if (hh + 2 <= hpg) batch(std::integral_constant<int, 2>{});
+      if (hh < hpg) batch(std::integral_constant<int, 1>{});
+      scores[row * n_keys + c] = acc;
+      const uint32_t o = float_ord(acc);
+      key[u] = descending ? ~o : o;  // smaller = better
+      if (force_first && c == 0) key[u] = 0u;
+    }
+  }
+  if (tid == 0) { s_prefix = 0u; s_need = (int)k; }
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    if (tid < 256) hist[tid] = 0;
+    __syncthreads();
+    const uint32_t prefix = s_prefix;
+    const int need = s_need;
+    const uint32_t pmask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      if (valid[u] && (key[u] & pmask) == prefix) atomicAdd(&hist[(key[u] >> shift) & 255], 1);
+    }
+    __syncthreads();
+    // the bin that holds the need-th smallest key: inclusive scan of the 256 bins by the first four waves
+    int mine = 0, incl = 0;
+    if (tid < 256) {
+      mine = hist[tid];
+      incl = mine;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int v = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += v;
+      }
+      if (lane == 63) scan_tot[wave] = incl;
+    }
+    __syncthreads();
+    if (tid < 256) {
+      for (int w = 0; w < wave; ++w) incl += scan_tot[w];
+      if (incl >= need && incl - mine < need) {  // exactly one thread
+        s_need = need - (incl - mine);
+        s_prefix = prefix | ((uint32_t)tid << shift);
+      }
+    }
+    __syncthreads();
+  }
+  const uint32_t kth = s_prefix;  // key of the k-th best element
+  const int need_eq = s_need;     // how many elements equal to kth are kept (lowest indices)
+  bool lt[2], eq[2];
+  int p_lt[2], p_eq[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    lt[u] = valid[u] && key[u] < kth;
+    eq[u] = valid[u] && key[u] == kth;
+    const unsigned long b_lt = __builtin_amdgcn_ballot_w64(lt[u]), b_eq = __builtin_amdgcn_ballot_w64(eq[u]);
+    const unsigned long below = (1ul << lane) - 1ul;
+    p_lt[u] = __builtin_popcountl(b_lt & below);
+    p_eq[u] = __builtin_popcountl(b_eq & below);
+    if (lane == 0) { seg_lt[u][wave] = __builtin_popcountl(b_lt); seg_eq[u][wave] = __builtin_popcountl(b_eq); }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    if (!lt[u] && !eq[u]) continue;
+    int b_lt = p_lt[u], b_eq = p_eq[u];  // kept-candidates with a lower index
+    for (int uu = 0; uu <= u; ++uu) {
+      const int wn = uu < u ? 16 : wave;
+      for (int w = 0; w < wn; ++w) { b_lt += seg_lt[uu][w]; b_eq += seg_eq[uu][w]; }
+    }
+    const long c = tid + 1024L * u;
+    if (lt[u]) out[row * k + b_lt + (b_eq < need_eq ? b_eq : need_eq)] = c;
+    else if (b_eq < need_eq) out[row * k + b_lt + b_eq] = c;
+  }
+}
+
 // votes[idx[i]] += 1 for every index inside [0, length); the counts are integers, so the order of the
 // additions does not matter
 __global__ __launch_bounds__(256) void vote_histogram_kernel(const long* __restrict__ idx, long n, long length,
@@ -532,6 +653,47 @@ extern "C" int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t 
     hipLaunchKernelGGL(evict_colsum_kernel<16>, dim3((unsigned)((n_keys + 15) / 16), (unsigned)n_chunks), dim3(256),
                        lds, st, probs, (long)n_heads, (long)n_queries, (long)n_keys, (long)heads_per_group, scores_out);
   }
+  return launch_status();
+}
+
+extern "C" int pdllm_evict_keep_from_probs(const float* probs, int64_t n_chunks, int64_t n_heads, int64_t n_queries,
+                                           int64_t n_keys, int64_t heads_per_group, int64_t capacity,
+                                           int32_t keep_high, int32_t force_keep_first, void* workspace,
+                                           int64_t workspace_bytes, float* scores_out, int64_t* indices_out,
+                                           pdllm_stream_t stream) {
+  if (!probs || !scores_out || !indices_out) return PDLLM_ERR_NULL;
+  if (n_chunks < 0 || n_heads <= 0 || n_queries <= 0 || n_keys <= 0 || heads_per_group <= 0 ||
+      n_heads % heads_per_group)
+    return PDLLM_ERR_SHAPE;
+  if (n_chunks == 0) return PDLLM_OK;
+  const int64_t n_groups = n_heads / heads_per_group;
+  int64_t keep = capacity < 1 ? 1 : capacity;
+  if (keep > n_keys) keep = n_keys;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const long blocks64 = (n_keys + 63) / 64 * n_chunks;
+  const bool two_launches = workspace != nullptr && blocks64 < 1024 && n_heads <= 65535 && n_chunks <= 65535 &&
+                            n_keys <= 2 * kSelThreads && n_chunks * n_groups <= 0x7fffffffL;
+  if (!two_launches) {
+    const int rc = pdllm_evict_colsum(probs, n_chunks, n_heads, n_queries, n_keys, heads_per_group, workspace,
+                                      workspace_bytes, scores_out, stream);
+    if (rc != PDLLM_OK) return rc;
+    return pdllm_topb_keep_bos(scores_out, n_chunks * n_groups, n_keys, n_keys, capacity, keep_high,
+                               force_keep_first, indices_out, stream);
+  }
+  if (workspace_bytes < n_chunks * n_heads * n_keys * 4 || ((uintptr_t)workspace % 4)) return PDLLM_ERR_WORKSPACE;
+  long parts = (512 + n_heads * n_chunks - 1) / (n_heads * n_chunks);
+  const long min_parts = (n_keys + 256 * kHeadsumCols - 1) / (256 * kHeadsumCols);
+  parts = parts < min_parts ? min_parts : parts;
+  const long width = (n_keys + parts - 1) / parts;
+  parts = (n_keys + width - 1) / width;
+  float* hsum = static_cast<float*>(workspace);
+  hipLaunchKernelGGL(evict_headsum_kernel, dim3((unsigned)parts, (unsigned)n_heads, (unsigned)n_chunks), dim3(256), 0,
+                     st, probs, (long)n_heads, (long)n_queries, (long)n_keys, width, hsum);
+  const int rc = launch_status();
+  if (rc != PDLLM_OK) return rc;
+  hipLaunchKernelGGL(evict_groupsum_select_kernel, dim3((unsigned)(n_chunks * n_groups)), dim3(kSelThreads), 0, st,
+                     hsum, (long)n_heads, (long)heads_per_group, (long)n_keys, (long)keep, keep_high ? 1 : 0,
+                     force_keep_first ? 1 : 0, scores_out, reinterpret_cast<long*>(indices_out));
   return launch_status();
 }
 

@@ -601,12 +601,27 @@ def evict_colsum(probs: torch.Tensor, heads_per_group: Optional[int] = None) -> 
 
 def evict_keep_from_probs(probs: torch.Tensor, capacity: int, heads_per_group: Optional[int] = None,
                           keep_high: bool = True, force_keep_first: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
-    """One eviction step from ready-made attention probabilities: evict_colsum followed by topb_keep_bos
-    (fastdllm_engine.py:1230-1322 summed over queries and heads, then :903-927).  probs [chunks, H, Q, K] fp32 ->
-    (scores [chunks, groups, K] fp32, keep indices [chunks * groups, keep] int64, ascending)."""
-    scores = evict_colsum(probs, heads_per_group)
-    c, g, nk = scores.shape
-    return scores, topb_keep_bos(scores.view(c * g, nk), capacity, keep_high, force_keep_first)
+    """One eviction step from ready-made attention probabilities in one library call: evict_colsum followed by
+    topb_keep_bos, same bits (fastdllm_engine.py:1230-1322 summed over queries and heads, then :903-927).
+    probs [chunks, H, Q, K] fp32 -> (scores [chunks, groups, K] fp32, keep indices [chunks * groups, keep] int64,
+    ascending)."""
+    _need_cuda(probs)
+    if probs.dim() == 3:
+        probs = probs.unsqueeze(0)
+    if probs.dtype != torch.float32 or not probs.is_contiguous():
+        raise ValueError("probs must be contiguous fp32 [chunks, heads, queries, keys]")
+    c, h, nq, nk = probs.shape
+    hpg = h if heads_per_group is None else heads_per_group
+    if hpg <= 0 or h % hpg:
+        raise ValueError(f"{h} heads do not split into groups of {hpg}")
+    keep = min(max(1, int(capacity)), nk)
+    scores = torch.empty((c, h // hpg, nk), dtype=torch.float32, device=probs.device)
+    idx = torch.empty((c * (h // hpg), keep), dtype=torch.int64, device=probs.device)
+    ws = _workspace(probs.device, int(lib.pdllm_evict_colsum_workspace_bytes(c, h, nk)))
+    check(lib.pdllm_evict_keep_from_probs(probs.data_ptr(), c, h, nq, nk, hpg, int(capacity), 1 if keep_high else 0,
+                                          1 if force_keep_first else 0, _ptr(ws), 0 if ws is None else ws.numel(),
+                                          scores.data_ptr(), idx.data_ptr(), _stream(probs)), "evict_keep_from_probs")
+    return scores, idx
 
 
 def query_to_chunk_attention_scores(q: torch.Tensor, k: torch.Tensor, *, prefix_len: int, chunk_len: int,

@@ -134,6 +134,39 @@ def test_topb_degenerate_branches(dev):
     assert got == ref_ops.select_positions_from_token_scores(s[:5], capacity=6, chunk_len=40).tolist()
 
 
+@pytest.mark.parametrize("shape", [(8, 28, 64, 1025, 28), (8, 28, 64, 1025, 7), (3, 8, 5, 2048, 2), (2, 4, 3, 1024, 4),
+                                   (5, 6, 7, 37, 3), (2, 4, 3, 2049, 2), (1, 2, 2, 1, 2)])
+def test_evict_keep_from_probs_equals_the_two_calls(dev, shape):
+    """One eviction step in one library call (fastdllm_engine.py:1230-1322 summed, then :903-927): the scores and the
+    keep indices must be the bits of evict_colsum followed by topb_keep_bos, and the indices those of the oracle's
+    selection on the same scores -- for one and several head groups, rows of 1 to 2049 keys (2049: the step falls
+    back to the launches of the two calls), both score orders, with and without the forced first position, keep
+    counts from 1 to the whole row, and rows in which most scores tie."""
+    ops = _ops()
+    c, h, nq, nk, hpg = shape
+    gen = torch.Generator().manual_seed(sum(shape))
+    probs = torch.rand(c, h, nq, nk, generator=gen)
+    probs[0] = torch.round(probs[0] * 4) / 4                       # chunk 0: few distinct values, many ties
+    if c > 1:
+        probs[1] = 0.125                                           # chunk 1: every score equal
+    dp = probs.to(dev)
+    caps = sorted({0, 1, 2, nk // 4, nk - 1, nk, nk + 5} & set(range(0, nk + 6)))
+    for cap in caps:
+        for keep_high, force in ((True, True), (False, True), (True, False), (False, False)):
+            sc, idx = ops.evict_keep_from_probs(dp, cap, hpg, keep_high=keep_high, force_keep_first=force)
+            sc2 = ops.evict_colsum(dp, hpg)
+            idx2 = ops.topb_keep_bos(sc2.view(-1, nk), cap, keep_high, force)
+            assert torch.equal(sc, sc2) and torch.equal(idx, idx2), (shape, cap, keep_high, force)
+    ref_sc = ref_ops.evict_colsum(probs, hpg)
+    assert torch.equal(sc.cpu(), ref_sc)
+    cap = max(1, nk // 4)
+    sc, idx = ops.evict_keep_from_probs(dp, cap, hpg)
+    rows = ref_sc.view(-1, nk)
+    for r in range(rows.shape[0]):
+        assert idx[r].cpu().tolist() == ref_ops.select_positions_from_token_scores(rows[r], capacity=cap,
+                                                                                   chunk_len=nk).tolist()
+
+
 def test_query_to_chunk_scores(dev):
     gen = torch.Generator().manual_seed(9)
     prefix, chunk, ql = 3, 300, 8
