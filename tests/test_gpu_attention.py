@@ -348,6 +348,7 @@ def test_chunk_prefill_block_diagonal(dev, causal):
     ([1025, 700, 64, 1, 333, 1024, 1000, 129] * 2, (28, 4), False),
     ([2000, 1950], (32, 32), True),                                        # MHA: a column spans two to three key tiles
     ([4100] * 2, (28, 4), True),                                           # few units: teams of 64 workgroups
+    ([700, 650, 600, 590], (28, 4), True),                                 # 16 units: teams of 32 workgroups
 ])
 def test_chunk_prefill_stream_kernel(dev, lens, heads, causal):
     """Large batches of chunks run on resident workgroups that stream through their columns
