@@ -702,6 +702,69 @@ def test_seeded_random_shapes_and_plans(dev):
         check(out, ref, what=f"case {i} {case.meta} plan {plan} mask {mode}")
 
 
+def test_prefill_layer_replays_from_a_hip_graph(dev):
+    """A prefill layer (rotary on Q and K with the paged store of K and V in one launch, then the chunk attention on
+    the resident-workgroup kernel) captured once and replayed three times with new activations in the same buffers,
+    with eager launches and synchronisations in between; every replay equals the eager result bit for bit and the
+    pages hold the rotated keys of that replay."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(77)
+    Hq, Hkv, dd, P = 28, 4, 128, 256
+    lens = [700, 650, 600, 590, 1025, 129, 64, 1]
+    n = sum(lens)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=dev)
+    assert "attn_prefill_stream_kernel" in ops.describe_prefill_plan(len(lens), Hq, Hkv, max(lens), n, True)
+    q = torch.empty(n, Hq, dd, dtype=torch.bfloat16, device=dev)
+    k = torch.empty(n, Hkv, dd, dtype=torch.bfloat16, device=dev)
+    v = torch.empty(n, Hkv, dd, dtype=torch.bfloat16, device=dev)
+    out = torch.empty_like(q)
+    pages = (n + P - 1) // P
+    kc = torch.zeros(pages, P, Hkv, dd, dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    page_ids = torch.randperm(pages, generator=gen).to(torch.int32).to(dev)
+    slots = ops.slot_mapping_from_pages(page_ids, n)
+    pos = torch.cat([torch.arange(l) for l in lens]).to(dev)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, dd, 2).float() / dd))
+    ang = torch.arange(max(lens)).float()[:, None] * inv[None, :]
+    cos_sin = torch.cat([ang.cos(), ang.sin()], dim=-1).to(dev)
+
+    def fill():
+        q.copy_(torch.randn(q.shape, generator=gen).to(torch.bfloat16))
+        k.copy_(torch.randn(k.shape, generator=gen).to(torch.bfloat16))
+        v.copy_(torch.randn(v.shape, generator=gen).to(torch.bfloat16))
+
+    def layer():
+        ops.rope_qk_store(q, k, v, pos, cos_sin, kc, vc, slots)
+        ops.chunk_prefill_attention(q, k, v, cu, max_seqlen=max(lens), causal=True, out=out)
+
+    fill()
+    q0, k0 = q.clone(), k.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer()                                  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    q.copy_(q0); k.copy_(k0)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        layer()
+    for rep in range(3):
+        fill()
+        q_in, k_in = q.clone(), k.clone()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got, got_k, got_q = out.clone(), ops.kv_gather(kc, page_ids, n), q.clone()
+        out.zero_(); kc.zero_()
+        q.copy_(q_in); k.copy_(k_in)             # the rotation is in place: start again from the same activations
+        layer()
+        torch.cuda.synchronize()
+        assert torch.equal(got_q, q) and torch.equal(got, out), rep
+        assert torch.equal(got_k, ops.kv_gather(kc, page_ids, n)) and torch.equal(got_k, k), rep
+    assert torch.isfinite(out.float()).all() and out.float().abs().max() > 0.1
+
+
 def test_decode_step_replays_from_a_hip_graph(dev):
     """The library allocates nothing and never synchronises, so a denoise step (slot-table build + the layers'
     attention and merge launches) can be captured once and replayed: three replays with new queries and a new chunk
