@@ -159,6 +159,14 @@ def test_evict_keep_from_probs_equals_the_two_calls(dev, shape):
             assert torch.equal(sc, sc2) and torch.equal(idx, idx2), (shape, cap, keep_high, force)
     ref_sc = ref_ops.evict_colsum(probs, hpg)
     assert torch.equal(sc.cpu(), ref_sc)
+    # a caller without a workspace gets the launches of the two calls: the same bits
+    from prefilling_dllm_amd._lib import lib, check
+    keep = min(max(1, nk // 3), nk)
+    sc3 = torch.empty_like(sc2)
+    idx3 = torch.empty((sc2.shape[0] * sc2.shape[1], keep), dtype=torch.int64, device=dev)
+    check(lib.pdllm_evict_keep_from_probs(dp.data_ptr(), c, h, nq, nk, hpg, nk // 3, 1, 1, None, 0, sc3.data_ptr(),
+                                          idx3.data_ptr(), torch.cuda.current_stream().cuda_stream), "no workspace")
+    assert torch.equal(sc3, sc2) and torch.equal(idx3, ops.topb_keep_bos(sc2.view(-1, nk), nk // 3, True, True))
     cap = max(1, nk // 4)
     sc, idx = ops.evict_keep_from_probs(dp, cap, hpg)
     rows = ref_sc.view(-1, nk)
