@@ -126,16 +126,26 @@ __device__ __forceinline__ void softmax_update(f32x16 (&S)[NKB], bf16x8 (&P)[NKB
 
 // BUF (software-pipelined variants only): the K/V copies are buffer loads with a 32-bit byte offset per
 // lane; the host selects it when every source tensor is smaller than 4 GiB.
-template <int KV_FP8, int J, bool BUF = false>
-__global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void attn_fwd_kernel(const AttnKParams p) {
-  constexpr int NW = J == 8 ? 8 : 4;        // wavefronts per workgroup
-  constexpr int kDmaGroups = 16 / NW;       // a tile is 16 groups of 4 rows; a wave copies this many of them
+// SPEC (fp8 pages): J waves with one row block each run the software-pipelined loop on bf16 tiles that three more
+// waves write: they fetch the fp8 rows two tiles ahead, dequantise them and store them into LDS in the layout the
+// direct copies produce.
+template <int KV_FP8, int J, bool BUF = false, bool SPEC = false>
+__global__ __launch_bounds__(SPEC ? 64 * (J + 3) : J == 8 ? 512 : 256, (SPEC || (KV_FP8 && J > 4)) ? 1 : 2) void attn_fwd_kernel(const AttnKParams p) {
+  static_assert(!SPEC || (KV_FP8 && !BUF && J >= 4 && J <= 5), "producer waves serve fp8 pages only");
+  constexpr int NW = SPEC ? J + 3 : J == 8 ? 8 : 4;  // wavefronts per workgroup
+  constexpr int kDmaGroups = SPEC ? 1 : 16 / NW;      // a tile is 16 groups of 4 rows; a wave copies this many of them
   constexpr bool HAS_A = J >= 4;
-  constexpr bool HAS_B = J != 4 && J != 8;
+  constexpr bool HAS_B = !SPEC && J != 4 && J != 8;
   constexpr int GS = (J == 1 || J == 5) ? 4 : (J == 2 || J == 6) ? 2 : 1;  // waves sharing a B block
-  constexpr bool QB_LDS = J == 5 || J == 6;  // Q of the shared block(s) lives in LDS, not in registers
+  constexpr bool QB_LDS = !SPEC && (J == 5 || J == 6);  // Q of the shared block(s) lives in LDS, not in registers
 
   __shared__ __attribute__((aligned(1024))) char lds[kMainBytes];
+  // SPEC: staging area of the three producer waves -- per wave three times six groups of 8 fp8 rows and two rows of
+  // page scales (K and V), and four rows of slots, all filled by direct-to-LDS copies
+  constexpr int kLead = 2;  // steps between the request of a tile's rows and their use
+  constexpr int kRing = kLead + 1;
+  constexpr int kStTile = 6 * 1024, kStScales = kRing * kStTile, kStSlots = kStScales + kRing * 512, kStBytes = kStSlots + 8 * 256;
+  __shared__ __attribute__((aligned(1024))) char stage[SPEC ? 3 * kStBytes : 16];
   __shared__ float s_ml[4][2][32];
   // dynamic part: Q fragments of the shared blocks (QB_LDS), then the dense-mask bit rows
   // [2][kMaxTok][kNKB] of an active tile (one bit per key; only with PDLLM_MASK_DENSE)
@@ -269,7 +279,7 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
   int srowA = 0, srowB = 0, ridxA = -1, ridxB = -1;
   auto load_q = [&](int blk, bf16x8 (&Q)[8], int& srow, int& ridx) __attribute__((always_inline)) {
     const int r = row0 + 32 * blk + l32e;
-    const bool valid = blk >= 0 && r < rows;
+    const bool valid = blk >= 0 && r < rows && (!SPEC || blk < J);
     const int rr = valid ? r : 0;
     const int tq = rr / G;
     const int g = rr - tq * G;
@@ -311,8 +321,9 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
   ntok = ntok < kMaxTok ? ntok : kMaxTok;
   auto build_mask = [&](int t, int par) __attribute__((always_inline)) {
     if (p.mask_mode != PDLLM_MASK_DENSE || t < Tc) return;
+    if (SPEC && wave >= J) return;  // (the producer waves never get here)
     const int a0 = (t - Tc) * kKT;
-    for (int idx = tid; idx < ntok * kNKB; idx += NW * 64) {
+    for (int idx = tid; idx < ntok * kNKB; idx += (SPEC ? J : NW) * 64) {
       const int tok = idx / kNKB, w = idx % kNKB;
       const uint8_t* mp = mask_base + (long)(tq_first + tok) * p.mask_stride + a0 + 32 * w;
       uint32_t bits = 0;
@@ -581,7 +592,7 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
   // nothing is inserted between its parts.  Between the PV steps runs the row maximum of tile
   // t + 1, so that an iteration over an unmasked tile starts with its maximum known.
   // ------------------------------------------------------------------------------------------
-  constexpr bool PIPELINED = (J == 4 || J == 8) && !KV_FP8;
+  constexpr bool PIPELINED = ((J == 4 || J == 8) && !KV_FP8) || SPEC;
   if constexpr (PIPELINED) {
     if (T0 < T1) {
       typedef __attribute__((ext_vector_type(8))) short s16x8;
@@ -657,6 +668,136 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
         else if (young == 2) lds_wait<2>(x);
         else if (young == 1) lds_wait<1>(x);
         else lds_wait<0>(x);
+      };
+
+      // ---- producer waves (SPEC) ----
+      // Tile u of a piece lives in buffer (u - T0) & 1, for K as for V.  A tile is eight groups of 8 rows for K and
+      // eight for V; a producer has six places: wave J takes groups 0-5 of K, wave J + 1 groups 0-5 of V, wave
+      // J + 2 groups 6, 7 of K and of V (its last two places repeat the first two and are not written).
+      // Everything a producer fetches goes into its staging area by direct-to-LDS copies, so nothing in flight
+      // sits in registers: the slots of tile u + 3 (one per lane), then, with the slots of tile u + 2 read back,
+      // the page scales of K and of V and the fp8 rows of tile u + 2 (lane l: 16 values of row 8 g + l / 8).  Then
+      // it reads tile u, requested two steps ago, dequantises it and stores it in the layout the bf16 copies
+      // produce.  A round trip to memory takes about as long as an iteration of the other waves: with one step of
+      // lead the producers held them up.
+      // The waits count memory operations, so every step issues the same nine, for tiles past the end of the
+      // prefix with the last prefix tile's addresses (never read).  Tiles of the active block are bf16 and are
+      // copied straight into the tile buffer in the step that would have written them.
+      const bool producer = SPEC && wave >= J;
+      const int pw = wave - J;
+      const bool pfetch = T0 < Tc;  // this piece has prefix tiles
+      int pu = T0;                  // the tile this producer writes next
+      int pset = 0;                 // (pu - T0) % 3: staging tile of its rows
+      const unsigned st_base = (unsigned)(size_t)stage + (pw > 0 ? pw : 0) * kStBytes;
+      char* const st_ptr = stage + (pw > 0 ? pw : 0) * kStBytes;
+      const int p_row = lane >> 3, p_f = lane & 7;
+      const char* pk_cache = static_cast<const char*>(p.k_cache) + (long)kvh * p.cache_head_stride + 16 * p_f;
+      const char* pv_cache = static_cast<const char*>(p.v_cache) + (long)kvh * p.cache_head_stride + 16 * p_f;
+      auto place_is_k = [&](int j) __attribute__((always_inline)) { return pw == 0 || (pw == 2 && (j & 2) == 0); };
+      auto place_group = [&](int j) __attribute__((always_inline)) { return pw < 2 ? j : 6 + (j & 1); };
+      auto lds_copy4 = [&](const void* src, char* dst) __attribute__((always_inline)) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)dst, 4, 0, 0);
+      };
+      auto lds_copy16 = [&](const void* src, char* dst) __attribute__((always_inline)) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+      };
+      auto prod_slots = [&](int v) __attribute__((always_inline)) {  // request the slots of tile v
+        const int vv = v < Tc ? v : Tc - 1;
+        lds_copy4(tbl + (long)vv * kKT + lane, st_ptr + kStSlots + ((v - T0) & 7) * 256);
+      };
+      // The third producer follows K's schedule, which runs one tile ahead of V's (iteration t of the other waves
+      // needs K(t+2) and V(t+1)): in the step of tile w its V places hold tile w - 1, in the first two steps T0.
+      auto v_tile = [&](int w) __attribute__((always_inline)) { return pw == 2 && w > T0 ? w - 1 : w; };
+      // request scales and rows for the step of tile w; the slots have landed.  set = (w - T0) % 3
+      auto prod_fetch = [&](int w, int set) __attribute__((always_inline)) {
+        const unsigned sbk = st_base + kStSlots + ((w - T0) & 7) * 256;
+        const unsigned sbv = st_base + kStSlots + ((v_tile(w) - T0) & 7) * 256;
+        int sl[8];
+        asm volatile("ds_read_b32 %0, %1" : "=v"(sl[6]) : "v"(sbk + 4 * lane) : "memory");
+        asm volatile("ds_read_b32 %0, %1" : "=v"(sl[7]) : "v"(sbv + 4 * lane) : "memory");
+#pragma unroll
+        for (int j = 0; j < 6; ++j)
+          asm volatile("ds_read_b32 %0, %1" : "=v"(sl[j]) : "v"((place_is_k(j) ? sbk : sbv) + 4 * (8 * place_group(j) + p_row)) : "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(sl[0]), "+v"(sl[1]), "+v"(sl[2]), "+v"(sl[3]), "+v"(sl[4]), "+v"(sl[5]), "+v"(sl[6]), "+v"(sl[7])
+                     :
+                     : "memory");
+        const long sh = (long)kvh * p.scale_head_stride;
+        lds_copy4(p.k_scale + (long)(sl[6] >> p.page_shift) * p.scale_page_stride + sh, st_ptr + kStScales + set * 512);
+        lds_copy4(p.v_scale + (long)(sl[7] >> p.page_shift) * p.scale_page_stride + sh, st_ptr + kStScales + set * 512 + 256);
+#pragma unroll
+        for (int j = 0; j < 6; ++j)
+          lds_copy16((place_is_k(j) ? pk_cache : pv_cache) + (long)sl[j] * p.cache_token_stride,
+                     st_ptr + set * kStTile + j * 1024);
+      };
+      // dequantise and store what was fetched for the step of tile w
+      auto prod_write = [&](int w, int set) __attribute__((always_inline)) {
+        const int wv = v_tile(w);
+        const int lim = T1 < Tc ? T1 : Tc;  // prefix tiles of this piece end here
+        if (w < lim || wv < lim) {
+          typedef unsigned u32v4 __attribute__((ext_vector_type(4)));
+          u32v4 d[6];
+          float sc[6];
+          const unsigned db = st_base + set * kStTile + 16 * lane, scb = st_base + kStScales + set * 512 + 4 * p_row;
+#pragma unroll
+          for (int j = 0; j < 6; ++j) {
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(d[j]) : "v"(db), "n"(j * 1024) : "memory");
+            asm volatile("ds_read_b32 %0, %1" : "=v"(sc[j]) : "v"(scb + (place_is_k(j) ? 0 : 256) + 32 * place_group(j)) : "memory");
+          }
+          asm volatile("s_waitcnt lgkmcnt(0)"
+                       : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]), "+v"(d[4]), "+v"(d[5]),
+                         "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]), "+v"(sc[4]), "+v"(sc[5])
+                       :
+                       : "memory");
+#pragma unroll
+          for (int j = 0; j < 6; ++j) {
+            if (pw == 2 && j >= 4) continue;
+            const int x = place_is_k(j) ? w : wv;
+            if (x >= lim) continue;
+            const int r16 = 8 * (j & 1) + p_row;  // row & 15: every place's group has the parity of the place
+            const unsigned r = lds_base + ((x - T0) & 1) * kBufBytes + (place_is_k(j) ? 0 : kTileBytes) +
+                               (8 * place_group(j) + p_row) * kRowBytes;
+            const uint4 lo = dequant_fp8x8(d[j].x, d[j].y, sc[j]), hi = dequant_fp8x8(d[j].z, d[j].w, sc[j]);
+            const u32v4 lov = {lo.x, lo.y, lo.z, lo.w}, hiv = {hi.x, hi.y, hi.z, hi.w};
+            asm volatile("ds_write_b128 %0, %1" : : "v"(r + (((2 * p_f) ^ swz(r16)) << 4)), "v"(lov) : "memory");
+            asm volatile("ds_write_b128 %0, %1" : : "v"(r + (((2 * p_f + 1) ^ swz(r16)) << 4)), "v"(hiv) : "memory");
+          }
+        }
+        if (pw < 2 && w >= Tc && w < T1) {
+          const __bf16* nb = pw == 0 ? p.k_new + (long)q0 * p.kn_stride : p.v_new + (long)q0 * p.vn_stride;
+          const long nstride = pw == 0 ? p.kn_stride : p.vn_stride;
+          const int a0 = (w - Tc) * kKT;
+          char* tp = lds + ((w - T0) & 1) * kBufBytes + (pw == 0 ? 0 : kTileBytes);
+#pragma unroll
+          for (int gg = 0; gg < 16; ++gg) {
+            const int row = 4 * gg + (lane >> 4);
+            const int a = a0 + row < Sa ? a0 + row : a0;  // padding rows copy a valid row; they are masked
+            const int ch = (lane & 15) ^ swz(row);
+            lds_copy16(nb + a * nstride + kvh * kD + 8 * ch, tp + gg * 1024);
+          }
+          asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // the copies have landed
+        }
+      };
+      // One step.  Memory operations in issue order: ... slots(u+2), rows(u+1) | slots(u+3), rows(u+2), where
+      // "rows" are two scale copies and six row copies: the slots of tile u + 2 have landed when at most the 8
+      // operations of rows(u+1) are outstanding, the rows of tile u when at most the 18 issued after them are.
+      auto prod_step = [&]() __attribute__((always_inline)) {
+        if (pfetch) {
+          asm volatile("s_waitcnt vmcnt(8)" : : : "memory");
+          prod_slots(pu + kLead + 1);
+          prod_fetch(pu + kLead, pset == 0 ? kLead : pset - 1);
+          asm volatile("s_waitcnt vmcnt(%0)" : : "n"(9 * kLead) : "memory");
+        }
+        prod_write(pu, pset);
+        ++pu;
+        pset = pset == kLead ? 0 : pset + 1;
+      };
+      // (waits for this wave's LDS stores only: what it has requested for later tiles stays in flight)
+      auto prod_barrier = [&]() __attribute__((always_inline)) {
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+        __builtin_amdgcn_s_barrier();
       };
 
       // one iteration: softmax of tile t (scores in Sc) interleaved with QK of tile t + 1 (into Sn),
@@ -775,17 +916,21 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
             t0 = u0;
             t1 = u1;
             if (stp + PF < NS) rdkp(kf[stp % PF], stp + PF, par_tag);
-            if ((stp & 1) == 1 && ((stp & 7) >> 1) < kDmaGroups) {
-              if (stp < 8) issue_v1(t + 1, PAR ^ 1, (stp & 7) >> 1, steady_tag);
-              else if (k_on) issue_k1(t + 2, PAR, (stp & 7) >> 1, steady_tag);
+            if constexpr (!SPEC) {
+              if ((stp & 1) == 1 && ((stp & 7) >> 1) < kDmaGroups) {
+                if (stp < 8) issue_v1(t + 1, PAR ^ 1, (stp & 7) >> 1, steady_tag);
+                else if (k_on) issue_k1(t + 2, PAR, (stp & 7) >> 1, steady_tag);
+              }
             }
             __builtin_amdgcn_sched_barrier(0);
           }
+          if constexpr (!SPEC) {
 #pragma unroll
-          for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
-          if (MODE == 1) load_slots_ctx(t + 3);
-          else if (MODE == 2) load_slots_new(t + 3);
-          else if (t + 3 < T1) load_slots(t + 3);
+            for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
+            if (MODE == 1) load_slots_ctx(t + 3);
+            else if (MODE == 2) load_slots_new(t + 3);
+            else if (t + 3 < T1) load_slots(t + 3);
+          }
         } else {
 #pragma unroll
           for (int stp = 0; stp < NS; ++stp) {
@@ -845,23 +990,44 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
 
       // ---- prologue: K(T0), V(T0); then K(T0+1) while QK(T0) runs unpipelined ----
       f32x16 SX[2];
-      load_slots(T0);
-#pragma unroll
-      for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
-      issue_k(T0, 0);
-      issue_v(T0, 0);
-      if (T0 + 1 < T1) load_slots(T0 + 1);
-      build_mask(T0, 0);
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      __syncthreads();
-      if (T0 + 1 < T1) issue_k(T0 + 1, 1);
-#pragma unroll
-      for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
-      if (T0 + 2 < T1) load_slots(T0 + 2);
 #pragma unroll
       for (int b = 0; b < 2; ++b)
 #pragma unroll
         for (int i = 0; i < 16; ++i) SX[b][i] = 0.f;
+      if (SPEC && producer) {
+        if (pfetch) {
+#pragma unroll
+          for (int i = 0; i <= kLead; ++i) prod_slots(pu + i);
+          asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+#pragma unroll
+          for (int i = 0; i < kLead; ++i) prod_fetch(pu + i, i);
+        }
+        // Step 0 writes tile T0 into buffer 0; step 1, not for the V producer, K(T0 + 1) into buffer 1 while the
+        // other waves compute the first scores; step 2 + i belongs to iteration T0 + i of the other waves and
+        // writes K(T0 + i + 2) or V(T0 + i + 1).  One barrier per step, as many as the other waves pass.
+        const int nsteps = T1 - T0 + 2;
+        for (int i = 0; i < nsteps; ++i) {
+          if (i != 1 || pw != 1) prod_step();
+          prod_barrier();
+        }
+      } else {
+      if constexpr (!SPEC) {
+        load_slots(T0);
+#pragma unroll
+        for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
+        issue_k(T0, 0);
+        issue_v(T0, 0);
+        if (T0 + 1 < T1) load_slots(T0 + 1);
+      }
+      build_mask(T0, 0);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+      if constexpr (!SPEC) {
+        if (T0 + 1 < T1) issue_k(T0 + 1, 1);
+#pragma unroll
+        for (int i = 0; i < kDmaGroups; ++i) nsv[i] = nslot[i];
+        if (T0 + 2 < T1) load_slots(T0 + 2);
+      }
       {
         bf16x8 kf[PF];
 #pragma unroll
@@ -939,6 +1105,7 @@ __global__ __launch_bounds__(J == 8 ? 512 : 256, (KV_FP8 && J > 4) ? 1 : 2) void
 #pragma unroll
           for (int db = 0; db < 4; ++db) va[r][db] -= kBufBytes;
       }
+      }  // the waves that own row blocks
     }
   } else
   if (T0 < T1) {
@@ -1460,7 +1627,7 @@ static AttnPlan compute_plan(const pdllm_attn_desc* d, bool prefill) {
     if (d->rows_per_group && d->rows_per_group != 32 * J) continue;
     // 5 and 6 row blocks need more than 256 registers (one workgroup per CU): on request, and for an fp8
     // cache (which has no 8-block kernel) when they hold all rows of a (request, KV head) in one column
-    // where 4 blocks would leave a second, mostly empty one (160 rows of an MHA layer: 322 us against 362)
+    // where 4 blocks would leave a second, mostly empty one (160 rows of an MHA layer: 250-265 us against 362)
     if (!d->rows_per_group && (J == 5 || J == 6) && !(fp8 && nblk > 4 && nblk <= J)) continue;
     if (J == 8 && fp8) continue;  // the 8-wave workgroup has no room for the fp8 staging registers
     if (J == 8 && prefill && !d->rows_per_group) continue;  // coarser causal staircase: measured slower
@@ -1717,6 +1884,9 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
   const bool buf = !fp8 && (plan.J == 4 || plan.J == 8) && small(d->n_tokens, d->kn_stride * 2) &&
                    small(d->n_tokens, d->vn_stride * 2) &&
                    (!has_cache || small(d->n_pages * (int64_t)d->page_size, d->cache_token_stride * 2));
+#ifndef PDLLM_FP8_PRODUCERS
+#define PDLLM_FP8_PRODUCERS 1
+#endif
 #define PDLLM_LAUNCH(JJ)                                                                              \
   do {                                                                                                \
     if (fp8) hipLaunchKernelGGL((attn_fwd_kernel<1, JJ>), grid, block, dyn, stream, p);               \
@@ -1729,7 +1899,11 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
       if (buf) hipLaunchKernelGGL((attn_fwd_kernel<0, 4, true>), grid, block, dyn, stream, p);
       else PDLLM_LAUNCH(4);
       break;
-    case 5: PDLLM_LAUNCH(5); break;
+    case 5:
+      if (fp8 && PDLLM_FP8_PRODUCERS)  // (no Q fragments in LDS: only the mask rows are dynamic)
+        hipLaunchKernelGGL((attn_fwd_kernel<1, 5, false, true>), grid, dim3(64 * 8), dyn_lds_bytes(4, d->mask_mode), stream, p);
+      else PDLLM_LAUNCH(5);
+      break;
     case 6: PDLLM_LAUNCH(6); break;
     case 8:
       if (fp8) PDLLM_LAUNCH(8);
