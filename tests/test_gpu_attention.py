@@ -499,6 +499,36 @@ def test_cache_beyond_four_gib_uses_wide_addresses(dev):
     del kc, vc
 
 
+def test_fp8_cache_beyond_four_gib_takes_the_register_staged_kernel(dev):
+    """Five row blocks on fp8 pages run with producer waves that address the caches with 32-bit offsets; a cache
+    of 4 GiB or more takes the kernel that dequantises through registers with 64-bit addresses.  The same
+    request through a small cache and through pages at the far end of a 4.3 GB cache: both match the oracle."""
+    ops = _ops()
+    case = configs.chunked_prefix_case(43, n_req=2, n_chunks=5, chunk_tokens=300, topk=3, q_len=150, Hq=8, Hkv=8,
+                                       fp8=True)
+    ref = oracle_case(case)
+    check(run_case(case, dev), ref, what="small cache")
+    n_small, page = case.k_cache.shape[0], case.k_cache.shape[1]
+    n_big = (1 << 32) // (page * 8 * 128) + 64      # pages of page x 8 heads x 128 bytes: a little over 4 GiB
+    shift = n_big - n_small
+    kc = torch.empty((n_big, page, 8, 128), dtype=case.k_cache.dtype, device=dev)
+    vc = torch.empty_like(kc)
+    kc[shift:] = case.k_cache.to(dev)
+    vc[shift:] = case.v_cache.to(dev)
+    ks = torch.ones((n_big,) + tuple(case.k_scale.shape[1:]), dtype=torch.float32, device=dev)
+    vs = torch.ones_like(ks)
+    ks[shift:] = case.k_scale.to(dev)
+    vs[shift:] = case.v_scale.to(dev)
+    rp, rs, rl, mr = case.range_tensors()
+    d = lambda t: t.to(dev)
+    out = ops.sparse_decode_attention(d(case.q), d(case.k_new), d(case.v_new), kc, vc,
+                                      d(case.block_table + shift), d(case.q_start_loc), max_q_len=case.max_q,
+                                      max_ctx_len=case.max_ctx, ranges=(d(rp), d(rs), d(rl), mr), k_scale=ks, v_scale=vs)
+    torch.cuda.synchronize()
+    check(out.float().cpu(), ref, what="4.3 GB cache")
+    del kc, vc
+
+
 def test_error_codes(dev):
     ops = _ops()
     q = torch.zeros(32, 4, 64, dtype=torch.bfloat16, device=dev)
