@@ -263,6 +263,189 @@ __global__ __launch_bounds__(SPEC ? 64 * (J + 3) : J == 8 ? 512 : 256, (SPEC || 
   const int T0 = tb < T ? tb : T;
   const int T1 = te < T ? te : T;
 
+  if constexpr (SPEC) {
+    if (wave >= J) {
+    // ---- producer waves (SPEC) ----
+    // Tile u of a piece lives in buffer (u - T0) & 1, for K as for V.  A tile is eight groups of 8 rows for K and
+    // eight for V: wave J takes groups 0-5 of K, wave J + 1 groups 0-5 of V, wave J + 2 groups 6, 7 of both.
+    // Everything a producer fetches goes into its staging area by direct-to-LDS copies, so nothing in flight
+    // sits in registers: the slots of tile u + 3 (one per lane), then, with the slots of tile u + 2 read back,
+    // its page scales and its fp8 rows (lane l: 16 values of row 8 g + l / 8).  Then it reads tile u, requested
+    // two steps ago, dequantises it and stores it in the layout the bf16 copies produce.
+    // The waits count memory operations, so every step issues the same number, for tiles past the end of the
+    // prefix with the last prefix tile's addresses (never read).  Tiles of the active block are bf16 and are
+    // copied straight into the tile buffer in the step that would have written them.
+    // (The launcher has checked that slots and strides fit 24-bit multiplies and the caches 32-bit offsets.)
+    auto lds_copy4 = [&](const void* src, char* dst) __attribute__((always_inline)) {
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)dst, 4, 0, 0);
+    };
+    auto lds_copy16 = [&](const void* src, char* dst) __attribute__((always_inline)) {
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    };
+    auto run_producer = [&](auto pw_tag) __attribute__((always_inline)) {
+      constexpr int PW = decltype(pw_tag)::value;
+      constexpr int NPL = PW == 2 ? 4 : 6;  // places: (tensor, group of 8 rows)
+      constexpr int NSC = PW == 2 ? 2 : 1;  // scale rows: K, V or both
+      constexpr int NF = NSC + NPL;         // copies of one tile's scales and rows
+      auto place_is_k = [](int j) { return PW == 0 || (PW == 2 && j < 2); };
+      auto place_group = [](int j) { return PW < 2 ? j : 6 + (j & 1); };
+      const bool pfetch = T0 < Tc;  // this piece has prefix tiles
+      int pu = T0;                  // the tile (of K's numbering) of the next step
+      int pset = 0;                 // (pu - T0) % kRing: staging tile of its rows
+      const unsigned st_base = (unsigned)(size_t)stage + PW * kStBytes;
+      char* const st_ptr = stage + PW * kStBytes;
+      // (lane coordinates made opaque per piece: as loop invariants of the kernel the addresses built on them would
+      // be spilled, and a reload waits for every copy in flight)
+      int lane_p = lane;
+      asm volatile("" : "+v"(lane_p));
+      const int p_row = lane_p >> 3, p_f = lane_p & 7;
+      const char* pk_cache = static_cast<const char*>(p.k_cache) + (long)kvh * p.cache_head_stride + 16 * p_f;
+      const char* pv_cache = static_cast<const char*>(p.v_cache) + (long)kvh * p.cache_head_stride + 16 * p_f;
+      const float* pk_scale = p.k_scale + (long)kvh * p.scale_head_stride;
+      const float* pv_scale = p.v_scale + (long)kvh * p.scale_head_stride;
+      const unsigned tstride = (unsigned)p.cache_token_stride, sstride = (unsigned)p.scale_page_stride * 4u;
+      auto prod_slots = [&](int v) __attribute__((always_inline)) {  // request the slots of tile v
+        const int vv = v < Tc ? v : Tc - 1;
+        lds_copy4(tbl + (long)vv * kKT + lane_p, st_ptr + kStSlots + ((v - T0) & 7) * 256);
+      };
+      // The third producer follows K's schedule, which runs one tile ahead of V's (iteration t of the other
+      // waves needs K(t+2) and V(t+1)): in the step of tile w its V places hold tile w - 1, in the first two
+      // steps T0.
+      auto v_tile = [&](int w) __attribute__((always_inline)) { return PW == 2 && w > T0 ? w - 1 : w; };
+      // request scales and rows for the step of tile w; the slots have landed.  set = (w - T0) % kRing
+      auto prod_fetch = [&](int w, int set) __attribute__((always_inline)) {
+        const unsigned sbk = st_base + kStSlots + ((w - T0) & 7) * 256;
+        const unsigned sbv = st_base + kStSlots + ((v_tile(w) - T0) & 7) * 256;
+        int sl[NPL], so[NSC];
+#pragma unroll
+        for (int i = 0; i < NSC; ++i)
+          asm volatile("ds_read_b32 %0, %1" : "=v"(so[i]) : "v"((i == 0 && PW != 1 ? sbk : sbv) + 4 * lane_p) : "memory");
+#pragma unroll
+        for (int j = 0; j < NPL; ++j)
+          asm volatile("ds_read_b32 %0, %1" : "=v"(sl[j]) : "v"((place_is_k(j) ? sbk : sbv) + 4 * (8 * place_group(j) + p_row)) : "memory");
+        if constexpr (PW == 2)
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sl[0]), "+v"(sl[1]), "+v"(sl[2]), "+v"(sl[3]), "+v"(so[0]), "+v"(so[1]) : : "memory");
+        else
+          asm volatile("s_waitcnt lgkmcnt(0)"
+                       : "+v"(sl[0]), "+v"(sl[1]), "+v"(sl[2]), "+v"(sl[3]), "+v"(sl[4]), "+v"(sl[5]), "+v"(so[0])
+                       :
+                       : "memory");
+#pragma unroll
+        for (int i = 0; i < NSC; ++i) {
+          const float* sp = (i == 0 && PW != 1) ? pk_scale : pv_scale;
+          lds_copy4(reinterpret_cast<const char*>(sp) + __umul24((unsigned)(so[i] >> p.page_shift), sstride),
+                    st_ptr + kStScales + set * 512 + i * 256);
+        }
+#pragma unroll
+        for (int j = 0; j < NPL; ++j)
+          lds_copy16((place_is_k(j) ? pk_cache : pv_cache) + __umul24((unsigned)sl[j], tstride),
+                     st_ptr + set * kStTile + j * 1024);
+      };
+      // dequantise and store what was fetched for the step of tile w
+      auto prod_write = [&](int w, int set) __attribute__((always_inline)) {
+        const int wv = v_tile(w);
+        const int lim = T1 < Tc ? T1 : Tc;  // prefix tiles of this piece end here
+        if (w < lim || wv < lim) {
+          typedef unsigned u32v4 __attribute__((ext_vector_type(4)));
+          u32v4 d[NPL];
+          float sc[NPL];
+          const unsigned db = st_base + set * kStTile + 16 * lane_p, scb = st_base + kStScales + set * 512 + 4 * p_row;
+#pragma unroll
+          for (int j = 0; j < NPL; ++j) {
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(d[j]) : "v"(db), "n"(j * 1024) : "memory");
+            // (scale row 0 is K's for the first and the third producer, V's for the second; row 1 is V's)
+            if (place_is_k(j) || PW == 1)
+              asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(sc[j]) : "v"(scb), "n"(32 * place_group(j)) : "memory");
+            else
+              asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(sc[j]) : "v"(scb), "n"(256 + 32 * place_group(j)) : "memory");
+          }
+          if constexpr (PW == 2)
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]), "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3])
+                         :
+                         : "memory");
+          else
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]), "+v"(d[4]), "+v"(d[5]),
+                           "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]), "+v"(sc[4]), "+v"(sc[5])
+                         :
+                         : "memory");
+#pragma unroll
+          for (int j = 0; j < NPL; ++j) {
+            const int x = place_is_k(j) ? w : wv;
+            if (x >= lim) continue;
+            const int r16 = 8 * (j & 1) + p_row;  // row & 15: every place's group has the parity of the place
+            const unsigned r = lds_base + ((x - T0) & 1) * kBufBytes + (place_is_k(j) ? 0 : kTileBytes) +
+                               (8 * place_group(j) + p_row) * kRowBytes;
+            const uint4 lo = dequant_fp8x8(d[j].x, d[j].y, sc[j]), hi = dequant_fp8x8(d[j].z, d[j].w, sc[j]);
+            const u32v4 lov = {lo.x, lo.y, lo.z, lo.w}, hiv = {hi.x, hi.y, hi.z, hi.w};
+            asm volatile("ds_write_b128 %0, %1" : : "v"(r + (((2 * p_f) ^ swz(r16)) << 4)), "v"(lov) : "memory");
+            asm volatile("ds_write_b128 %0, %1" : : "v"(r + (((2 * p_f + 1) ^ swz(r16)) << 4)), "v"(hiv) : "memory");
+          }
+        }
+        if (PW < 2 && w >= Tc && w < T1) {
+          const __bf16* nb = PW == 0 ? p.k_new + (long)q0 * p.kn_stride : p.v_new + (long)q0 * p.vn_stride;
+          const long nstride = PW == 0 ? p.kn_stride : p.vn_stride;
+          const int a0 = (w - Tc) * kKT;
+          char* tp = lds + ((w - T0) & 1) * kBufBytes + (PW == 0 ? 0 : kTileBytes);
+#pragma unroll
+          for (int gg = 0; gg < 16; ++gg) {
+            const int row = 4 * gg + (lane_p >> 4);
+            const int a = a0 + row < Sa ? a0 + row : a0;  // padding rows copy a valid row; they are masked
+            const int ch = (lane_p & 15) ^ swz(row);
+            lds_copy16(nb + a * nstride + kvh * kD + 8 * ch, tp + gg * 1024);
+          }
+          asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // the copies have landed
+        }
+      };
+      if (pfetch) {
+#pragma unroll
+        for (int i = 0; i <= kLead; ++i) prod_slots(pu + i);
+        asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+#pragma unroll
+        for (int i = 0; i < kLead; ++i) prod_fetch(pu + i, i);
+      }
+      // Step 0 writes tile T0 into buffer 0; step 1, not for the V producer, K(T0 + 1) into buffer 1 while the
+      // other waves compute the first scores; step 2 + i belongs to iteration T0 + i of the other waves and
+      // writes K(T0 + i + 2) or V(T0 + i + 1).  One barrier per step, as many as the other waves pass.
+      // Memory operations in issue order: ... slots(u+2), rows(u+1) | slots(u+3), rows(u+2), "rows" being the
+      // NF copies of scales and rows: the slots of tile u + 2 have landed when at most the NF operations of
+      // rows(u+1) are outstanding, the rows of tile u when at most the kLead (NF + 1) issued after them are.
+      const int nsteps = T1 - T0 + 2;
+      for (int i = 0; i < nsteps; ++i) {
+        if (i != 1 || PW != 1) {
+          if (pfetch) {
+            asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NF) : "memory");
+            prod_slots(pu + kLead + 1);
+            prod_fetch(pu + kLead, pset == 0 ? kLead : pset - 1);
+            asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kLead * (NF + 1)) : "memory");
+          }
+          prod_write(pu, pset);
+          ++pu;
+          pset = pset == kLead ? 0 : pset + 1;
+        }
+        // (waits for this wave's LDS stores only: what it has requested for later tiles stays in flight)
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+        __builtin_amdgcn_s_barrier();
+      }
+    };
+
+      if (T0 < T1) {
+        if (wave == J) run_producer(std::integral_constant<int, 0>{});
+        else if (wave == J + 1) run_producer(std::integral_constant<int, 1>{});
+        else run_producer(std::integral_constant<int, 2>{});
+      }
+      if (head_rt >= 0 || y < y_end) {  // (the barrier between two pieces, as at the end of this loop)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+      }
+      continue;
+    }
+  }
+
   // ---- row blocks of this wave ----
   const int blkA = wave;
   const int gi = wave & (GS - 1);  // index of this wave among the GS waves sharing its B block
@@ -670,170 +853,6 @@ __global__ __launch_bounds__(SPEC ? 64 * (J + 3) : J == 8 ? 512 : 256, (SPEC || 
         else lds_wait<0>(x);
       };
 
-      // ---- producer waves (SPEC) ----
-      // Tile u of a piece lives in buffer (u - T0) & 1, for K as for V.  A tile is eight groups of 8 rows for K and
-      // eight for V: wave J takes groups 0-5 of K, wave J + 1 groups 0-5 of V, wave J + 2 groups 6, 7 of both.
-      // Everything a producer fetches goes into its staging area by direct-to-LDS copies, so nothing in flight
-      // sits in registers: the slots of tile u + 3 (one per lane), then, with the slots of tile u + 2 read back,
-      // its page scales and its fp8 rows (lane l: 16 values of row 8 g + l / 8).  Then it reads tile u, requested
-      // two steps ago, dequantises it and stores it in the layout the bf16 copies produce.
-      // The waits count memory operations, so every step issues the same number, for tiles past the end of the
-      // prefix with the last prefix tile's addresses (never read).  Tiles of the active block are bf16 and are
-      // copied straight into the tile buffer in the step that would have written them.
-      // (The launcher has checked that slots and strides fit 24-bit multiplies and the caches 32-bit offsets.)
-      const bool producer = SPEC && wave >= J;
-      auto lds_copy4 = [&](const void* src, char* dst) __attribute__((always_inline)) {
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (__attribute__((address_space(3))) void*)dst, 4, 0, 0);
-      };
-      auto lds_copy16 = [&](const void* src, char* dst) __attribute__((always_inline)) {
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-      };
-      auto run_producer = [&](auto pw_tag) __attribute__((always_inline)) {
-        constexpr int PW = decltype(pw_tag)::value;
-        constexpr int NPL = PW == 2 ? 4 : 6;  // places: (tensor, group of 8 rows)
-        constexpr int NSC = PW == 2 ? 2 : 1;  // scale rows: K, V or both
-        constexpr int NF = NSC + NPL;         // copies of one tile's scales and rows
-        auto place_is_k = [](int j) { return PW == 0 || (PW == 2 && j < 2); };
-        auto place_group = [](int j) { return PW < 2 ? j : 6 + (j & 1); };
-        const bool pfetch = T0 < Tc;  // this piece has prefix tiles
-        int pu = T0;                  // the tile (of K's numbering) of the next step
-        int pset = 0;                 // (pu - T0) % kRing: staging tile of its rows
-        const unsigned st_base = (unsigned)(size_t)stage + PW * kStBytes;
-        char* const st_ptr = stage + PW * kStBytes;
-        const int p_row = lane >> 3, p_f = lane & 7;
-        const char* pk_cache = static_cast<const char*>(p.k_cache) + (long)kvh * p.cache_head_stride + 16 * p_f;
-        const char* pv_cache = static_cast<const char*>(p.v_cache) + (long)kvh * p.cache_head_stride + 16 * p_f;
-        const float* pk_scale = p.k_scale + (long)kvh * p.scale_head_stride;
-        const float* pv_scale = p.v_scale + (long)kvh * p.scale_head_stride;
-        const unsigned tstride = (unsigned)p.cache_token_stride, sstride = (unsigned)p.scale_page_stride * 4u;
-        auto prod_slots = [&](int v) __attribute__((always_inline)) {  // request the slots of tile v
-          const int vv = v < Tc ? v : Tc - 1;
-          lds_copy4(tbl + (long)vv * kKT + lane, st_ptr + kStSlots + ((v - T0) & 7) * 256);
-        };
-        // The third producer follows K's schedule, which runs one tile ahead of V's (iteration t of the other
-        // waves needs K(t+2) and V(t+1)): in the step of tile w its V places hold tile w - 1, in the first two
-        // steps T0.
-        auto v_tile = [&](int w) __attribute__((always_inline)) { return PW == 2 && w > T0 ? w - 1 : w; };
-        // request scales and rows for the step of tile w; the slots have landed.  set = (w - T0) % kRing
-        auto prod_fetch = [&](int w, int set) __attribute__((always_inline)) {
-          const unsigned sbk = st_base + kStSlots + ((w - T0) & 7) * 256;
-          const unsigned sbv = st_base + kStSlots + ((v_tile(w) - T0) & 7) * 256;
-          int sl[NPL], so[NSC];
-#pragma unroll
-          for (int i = 0; i < NSC; ++i)
-            asm volatile("ds_read_b32 %0, %1" : "=v"(so[i]) : "v"((i == 0 && PW != 1 ? sbk : sbv) + 4 * lane) : "memory");
-#pragma unroll
-          for (int j = 0; j < NPL; ++j)
-            asm volatile("ds_read_b32 %0, %1" : "=v"(sl[j]) : "v"((place_is_k(j) ? sbk : sbv) + 4 * (8 * place_group(j) + p_row)) : "memory");
-          if constexpr (PW == 2)
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sl[0]), "+v"(sl[1]), "+v"(sl[2]), "+v"(sl[3]), "+v"(so[0]), "+v"(so[1]) : : "memory");
-          else
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(sl[0]), "+v"(sl[1]), "+v"(sl[2]), "+v"(sl[3]), "+v"(sl[4]), "+v"(sl[5]), "+v"(so[0])
-                         :
-                         : "memory");
-#pragma unroll
-          for (int i = 0; i < NSC; ++i) {
-            const float* sp = (i == 0 && PW != 1) ? pk_scale : pv_scale;
-            lds_copy4(reinterpret_cast<const char*>(sp) + __umul24((unsigned)(so[i] >> p.page_shift), sstride),
-                      st_ptr + kStScales + set * 512 + i * 256);
-          }
-#pragma unroll
-          for (int j = 0; j < NPL; ++j)
-            lds_copy16((place_is_k(j) ? pk_cache : pv_cache) + __umul24((unsigned)sl[j], tstride),
-                       st_ptr + set * kStTile + j * 1024);
-        };
-        // dequantise and store what was fetched for the step of tile w
-        auto prod_write = [&](int w, int set) __attribute__((always_inline)) {
-          const int wv = v_tile(w);
-          const int lim = T1 < Tc ? T1 : Tc;  // prefix tiles of this piece end here
-          if (w < lim || wv < lim) {
-            typedef unsigned u32v4 __attribute__((ext_vector_type(4)));
-            u32v4 d[NPL];
-            float sc[NPL];
-            const unsigned db = st_base + set * kStTile + 16 * lane, scb = st_base + kStScales + set * 512 + 4 * p_row;
-#pragma unroll
-            for (int j = 0; j < NPL; ++j) {
-              asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(d[j]) : "v"(db), "n"(j * 1024) : "memory");
-              // (scale row 0 is K's for the first and the third producer, V's for the second; row 1 is V's)
-              if (place_is_k(j) || PW == 1)
-                asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(sc[j]) : "v"(scb), "n"(32 * place_group(j)) : "memory");
-              else
-                asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(sc[j]) : "v"(scb), "n"(256 + 32 * place_group(j)) : "memory");
-            }
-            if constexpr (PW == 2)
-              asm volatile("s_waitcnt lgkmcnt(0)"
-                           : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]), "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3])
-                           :
-                           : "memory");
-            else
-              asm volatile("s_waitcnt lgkmcnt(0)"
-                           : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]), "+v"(d[4]), "+v"(d[5]),
-                             "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]), "+v"(sc[4]), "+v"(sc[5])
-                           :
-                           : "memory");
-#pragma unroll
-            for (int j = 0; j < NPL; ++j) {
-              const int x = place_is_k(j) ? w : wv;
-              if (x >= lim) continue;
-              const int r16 = 8 * (j & 1) + p_row;  // row & 15: every place's group has the parity of the place
-              const unsigned r = lds_base + ((x - T0) & 1) * kBufBytes + (place_is_k(j) ? 0 : kTileBytes) +
-                                 (8 * place_group(j) + p_row) * kRowBytes;
-              const uint4 lo = dequant_fp8x8(d[j].x, d[j].y, sc[j]), hi = dequant_fp8x8(d[j].z, d[j].w, sc[j]);
-              const u32v4 lov = {lo.x, lo.y, lo.z, lo.w}, hiv = {hi.x, hi.y, hi.z, hi.w};
-              asm volatile("ds_write_b128 %0, %1" : : "v"(r + (((2 * p_f) ^ swz(r16)) << 4)), "v"(lov) : "memory");
-              asm volatile("ds_write_b128 %0, %1" : : "v"(r + (((2 * p_f + 1) ^ swz(r16)) << 4)), "v"(hiv) : "memory");
-            }
-          }
-          if (PW < 2 && w >= Tc && w < T1) {
-            const __bf16* nb = PW == 0 ? p.k_new + (long)q0 * p.kn_stride : p.v_new + (long)q0 * p.vn_stride;
-            const long nstride = PW == 0 ? p.kn_stride : p.vn_stride;
-            const int a0 = (w - Tc) * kKT;
-            char* tp = lds + ((w - T0) & 1) * kBufBytes + (PW == 0 ? 0 : kTileBytes);
-#pragma unroll
-            for (int gg = 0; gg < 16; ++gg) {
-              const int row = 4 * gg + (lane >> 4);
-              const int a = a0 + row < Sa ? a0 + row : a0;  // padding rows copy a valid row; they are masked
-              const int ch = (lane & 15) ^ swz(row);
-              lds_copy16(nb + a * nstride + kvh * kD + 8 * ch, tp + gg * 1024);
-            }
-            asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // the copies have landed
-          }
-        };
-        if (pfetch) {
-#pragma unroll
-          for (int i = 0; i <= kLead; ++i) prod_slots(pu + i);
-          asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
-#pragma unroll
-          for (int i = 0; i < kLead; ++i) prod_fetch(pu + i, i);
-        }
-        // Step 0 writes tile T0 into buffer 0; step 1, not for the V producer, K(T0 + 1) into buffer 1 while the
-        // other waves compute the first scores; step 2 + i belongs to iteration T0 + i of the other waves and
-        // writes K(T0 + i + 2) or V(T0 + i + 1).  One barrier per step, as many as the other waves pass.
-        // Memory operations in issue order: ... slots(u+2), rows(u+1) | slots(u+3), rows(u+2), "rows" being the
-        // NF copies of scales and rows: the slots of tile u + 2 have landed when at most the NF operations of
-        // rows(u+1) are outstanding, the rows of tile u when at most the kLead (NF + 1) issued after them are.
-        const int nsteps = T1 - T0 + 2;
-        for (int i = 0; i < nsteps; ++i) {
-          if (i != 1 || PW != 1) {
-            if (pfetch) {
-              asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NF) : "memory");
-              prod_slots(pu + kLead + 1);
-              prod_fetch(pu + kLead, pset == 0 ? kLead : pset - 1);
-              asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kLead * (NF + 1)) : "memory");
-            }
-            prod_write(pu, pset);
-            ++pu;
-            pset = pset == kLead ? 0 : pset + 1;
-          }
-          // (waits for this wave's LDS stores only: what it has requested for later tiles stays in flight)
-          asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-          __builtin_amdgcn_s_barrier();
-        }
-      };
-
       // one iteration: softmax of tile t (scores in Sc) interleaved with QK of tile t + 1 (into Sn),
       // then PV of tile t.  PAR = buffer of V(t); K(t+1) sits in the other buffer.
       int flip = kBufBytes;  // ka: buffer 1 -> 0 -> 1 ..., va: buffer 0 -> 1 -> 0 ...
@@ -1028,11 +1047,6 @@ __global__ __launch_bounds__(SPEC ? 64 * (J + 3) : J == 8 ? 512 : 256, (SPEC || 
       for (int b = 0; b < 2; ++b)
 #pragma unroll
         for (int i = 0; i < 16; ++i) SX[b][i] = 0.f;
-      if (SPEC && producer) {
-        if (wave == J) run_producer(std::integral_constant<int, 0>{});
-        else if (wave == J + 1) run_producer(std::integral_constant<int, 1>{});
-        else run_producer(std::integral_constant<int, 2>{});
-      } else {
       if constexpr (!SPEC) {
         load_slots(T0);
 #pragma unroll
@@ -1127,7 +1141,6 @@ __global__ __launch_bounds__(SPEC ? 64 * (J + 3) : J == 8 ? 512 : 256, (SPEC || 
 #pragma unroll
           for (int db = 0; db < 4; ++db) va[r][db] -= kBufBytes;
       }
-      }  // the waves that own row blocks
     }
   } else
   if (T0 < T1) {
