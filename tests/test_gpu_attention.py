@@ -283,6 +283,25 @@ def test_fp8_groups_of_five_and_six_row_blocks(dev, q_len, Hq, Hkv, blocks):
         check(run_case(case, dev, rows_per_group=32 * blocks, num_splits=splits), ref, what=f"splits={splits}")
 
 
+@pytest.mark.parametrize("plan", [dict(), dict(num_splits=2), dict(tiles_per_workgroup=7), dict(tiles_per_workgroup=1)],
+                         ids=["default", "split2", "span7", "span1"])
+def test_fp8_five_row_blocks_masks_and_ragged_pieces(dev, plan):
+    """The fp8 kernel for five row blocks has waves that only fill the tile buffers for the others: causal and
+    dense masks over the active block, 150 rows (the last row block and the last active tile ragged), prefixes that
+    end inside a tile, and workgroups whose span covers pieces of two columns or a single tile."""
+    case = configs.chunked_prefix_case(57, n_req=3, n_chunks=4, chunk_tokens=210, topk=2, q_len=150, Hq=4, Hkv=4,
+                                       fp8=True, shared_prefix=False)
+    check(run_case(case, dev, rows_per_group=160, **plan), oracle_case(case), what="full")
+    check(run_case(case, dev, rows_per_group=160, mask_mode="causal", **plan), oracle_case(case, mask_mode="causal"),
+          what="causal")
+    gen = torch.Generator().manual_seed(3)
+    n = case.q.shape[0]
+    mask = torch.rand(n, n, generator=gen) < 0.5
+    mask |= torch.eye(n, dtype=torch.bool)
+    check(run_case(case, dev, rows_per_group=160, mask_mode="dense", mask=mask, **plan),
+          oracle_case(case, mask_mode="dense", mask=mask), what="dense")
+
+
 def test_fp8_codes_decode_like_torch(dev):
     """All 256 e4m3 codes through the kernel's dequantisation == torch.float8_e4m3fn -> float."""
     ops = _ops()
