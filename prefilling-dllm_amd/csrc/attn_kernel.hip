@@ -1640,6 +1640,21 @@ static int compute_units() {
   return cached[dev];
 }
 
+#ifndef PDLLM_FP8_PRODUCERS
+#define PDLLM_FP8_PRODUCERS 1
+#endif
+// 32-bit copy offsets: a tensor the copies read is smaller than 4 GiB and its rows and row indices fit the 24-bit
+// multiply
+static bool small_tensor(int64_t rows, int64_t row_bytes) {
+  return rows < (1l << 24) && row_bytes < (1l << 24) && rows * row_bytes < (1l << 32) - 4096;
+}
+
+// fp8 pages, five row blocks: the kernel with producer waves addresses caches and scales with 32-bit offsets
+static bool fp8_producers_fit(const pdllm_attn_desc* d) {
+  return small_tensor(d->n_pages * (int64_t)d->page_size, d->cache_token_stride) &&
+         small_tensor(d->n_pages, d->scale_page_stride * 4);
+}
+
 static AttnPlan compute_plan(const pdllm_attn_desc* d, bool prefill) {
   const int G = d->num_q_heads / d->num_kv_heads;
   const long rows = (long)d->max_q_len * G;
@@ -1648,6 +1663,7 @@ static AttnPlan compute_plan(const pdllm_attn_desc* d, bool prefill) {
   const long T = (ctx + kKT - 1) / kKT + (d->max_q_len + kKT - 1) / kKT;
   const long units = (long)d->n_req * d->num_kv_heads;
   const bool fp8 = !prefill && d->k_cache != nullptr && d->max_ctx_len > 0 && d->kv_dtype == PDLLM_KV_FP8_E4M3;
+  const bool producers = fp8 && PDLLM_FP8_PRODUCERS && fp8_producers_fit(d);
   const int cus = compute_units();
   // kPiece: what a piece costs outside its tile loop (three round trips to memory before the first MFMA, the
   // last PV, the partial rows): about 3.2 tiles of a 4-wave workgroup
@@ -1662,8 +1678,17 @@ static AttnPlan compute_plan(const pdllm_attn_desc* d, bool prefill) {
     if (d->rows_per_group && d->rows_per_group != 32 * J) continue;
     // 5 and 6 row blocks need more than 256 registers (one workgroup per CU): on request, and for an fp8
     // cache (which has no 8-block kernel) when they hold all rows of a (request, KV head) in one column
-    // where 4 blocks would leave a second, mostly empty one (160 rows of an MHA layer: 250-265 us against 362)
-    if (!d->rows_per_group && (J == 5 || J == 6) && !(fp8 && nblk > 4 && nblk <= J)) continue;
+    // where 4 blocks would leave a second, mostly empty one (160 rows of an MHA layer: 250-265 us against 362).
+    // Five blocks with producer waves are a candidate for any fp8 shape of five blocks or more: per row block
+    // and tile they take 0.92 of what a pair of 4-block workgroups takes (8 x 1120 rows over 4096 keys, GQA 28/4:
+    // 116 against 122 us; 4 x 640 rows over 16400 keys, GQA 32/8: 227 against 237 us).
+    // -- where groups of five do not leave more empty row blocks than groups of four (7 blocks of a 32-row decode
+    // with GQA 28/4 are 5 + 2 against 4 + 3: 43.6 against 40.0 us).
+    const bool fives_fill = (nblk + 4) / 5 * 5 <= (nblk + 3) / 4 * 4;
+    if (!d->rows_per_group && (J == 5 || J == 6) &&
+        !(fp8 && nblk > 4 && (nblk <= J || (J == 5 && producers && fives_fill))))
+      continue;
+    const double units_per_wave = (J == 5 && producers) ? 0.66 : upw[ji];
     if (J == 8 && fp8) continue;  // the 8-wave workgroup has no room for the fp8 staging registers
     if (J == 8 && prefill && !d->rows_per_group) continue;  // coarser causal staircase: measured slower
     const long row_tiles = (nblk + J - 1) / J;
@@ -1702,7 +1727,7 @@ static AttnPlan compute_plan(const pdllm_attn_desc* d, bool prefill) {
         // spans and handle two or three pieces each.  The head is made `extra` tiles longer than a span; which
         // `extra` gives the shortest longest workgroup depends on where the cuts fall in the columns (a cut that
         // coincides with the end of a column saves a piece), so the candidates are laid out and compared.
-        const double tile_cost = kFixed + upw[ji], piece_cost = kPiece;
+        const double tile_cost = kFixed + units_per_wave, piece_cost = kPiece;
         double best_load = 1e300;
         long best_span = 0, best_head = 0;
         for (long extra = 0; extra <= 12; ++extra) {
@@ -1750,7 +1775,7 @@ static AttnPlan compute_plan(const pdllm_attn_desc* d, bool prefill) {
       }
       // the most loaded workgroup: its tiles and its pieces (two where the cuts do not respect the columns)
       const double wg_load = head > 0 ? set_load
-                                      : (double)span * (kFixed + upw[ji]) + kPiece * (cut && t_lin % span ? 2.0 : 1.0);
+                                      : (double)span * (kFixed + units_per_wave) + kPiece * (cut && t_lin % span ? 2.0 : 1.0);
       double cost = serial * wg_load + 1.0;
       if (cut) {
         // partial rows written and read back (~4 MB per unit of time), plus the merge launch
@@ -1911,17 +1936,10 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
   const bool fp8 = has_cache && d->kv_dtype == PDLLM_KV_FP8_E4M3;
   const int dyn = dyn_lds_bytes(plan.J, d->mask_mode);
   const dim3 grid((unsigned)plan.grid), block(plan.J == 8 && fp8 ? 512 : kThreads);
-  // 32-bit copy offsets: every tensor the copies read is smaller than 4 GiB and its rows and row
-  // indices fit the 24-bit multiply
-  const auto small = [](int64_t rows, int64_t row_bytes) {
-    return rows < (1l << 24) && row_bytes < (1l << 24) && rows * row_bytes < (1l << 32) - 4096;
-  };
+  const auto small = small_tensor;
   const bool buf = !fp8 && (plan.J == 4 || plan.J == 8) && small(d->n_tokens, d->kn_stride * 2) &&
                    small(d->n_tokens, d->vn_stride * 2) &&
                    (!has_cache || small(d->n_pages * (int64_t)d->page_size, d->cache_token_stride * 2));
-#ifndef PDLLM_FP8_PRODUCERS
-#define PDLLM_FP8_PRODUCERS 1
-#endif
 #define PDLLM_LAUNCH(JJ)                                                                              \
   do {                                                                                                \
     if (fp8) hipLaunchKernelGGL((attn_fwd_kernel<1, JJ>), grid, block, dyn, stream, p);               \
@@ -1935,8 +1953,7 @@ static int launch_attn(const pdllm_attn_desc* d, bool prefill, hipStream_t strea
       else PDLLM_LAUNCH(4);
       break;
     case 5:
-      if (fp8 && PDLLM_FP8_PRODUCERS && small(d->n_pages * (int64_t)d->page_size, d->cache_token_stride) &&
-          small(d->n_pages, d->scale_page_stride * 4))  // (no Q fragments in LDS: only the mask rows are dynamic)
+      if (fp8 && PDLLM_FP8_PRODUCERS && fp8_producers_fit(d))  // (no Q fragments in LDS: only the mask rows are dynamic)
         hipLaunchKernelGGL((attn_fwd_kernel<1, 5, false, true>), grid, dim3(64 * 8), dyn_lds_bytes(4, d->mask_mode), stream, p);
       else PDLLM_LAUNCH(5);
       break;

@@ -302,6 +302,35 @@ def test_fp8_five_row_blocks_masks_and_ragged_pieces(dev, plan):
           oracle_case(case, mask_mode="dense", mask=mask), what="dense")
 
 
+@pytest.mark.parametrize("q_len,Hq,Hkv,mode", [(160, 28, 4, "full"), (80, 8, 2, "causal"), (75, 8, 4, "full")])
+def test_fp8_default_plan_takes_groups_of_five_where_they_fill(dev, q_len, Hq, Hkv, mode):
+    """With fp8 pages the planner cuts the rows of a (request, KV head) into groups of five row blocks (the kernel
+    with producer waves) when that leaves no more empty blocks than groups of four: 35 blocks (7 groups), 10 blocks
+    (2 groups), 10 blocks with a ragged last one.  Several row groups per (request, KV head), by default and forced."""
+    ops = _ops()
+    case = configs.chunked_prefix_case(71 + q_len, n_req=2, n_chunks=5, chunk_tokens=300, topk=3, q_len=q_len,
+                                       Hq=Hq, Hkv=Hkv, fp8=True, shared_prefix=False)
+    d = lambda t: t.to(dev)
+    rp, rs, rl, mr = case.range_tensors()
+    pr = ops.PreparedAttention(d(case.q), d(case.k_new), d(case.v_new), d(case.k_cache), d(case.v_cache),
+                               d(case.block_table), d(case.q_start_loc), max_q_len=case.max_q, max_ctx_len=case.max_ctx,
+                               ranges=(d(rp), d(rs), d(rl), mr), k_scale=d(case.k_scale), v_scale=d(case.v_scale),
+                               mask_mode=mode)
+    if Hq == 28:  # (the smaller shapes take shorter row groups by default, to fill the compute units)
+        assert "kv=fp8 row_blocks=5" in pr.describe_plan(), pr.describe_plan()
+    ref = oracle_case(case, mask_mode=mode)
+    check(run_case(case, dev, mask_mode=mode), ref, what="default plan")
+    check(run_case(case, dev, mask_mode=mode, rows_per_group=160), ref, what="groups of 160 rows")
+    # 7 row blocks (32 response rows of 7 query heads each) stay with groups of four
+    small = configs.chunked_prefix_case(72, n_req=2, n_chunks=5, chunk_tokens=300, topk=3, q_len=32, fp8=True)
+    rp, rs, rl, mr = small.range_tensors()
+    pr = ops.PreparedAttention(d(small.q), d(small.k_new), d(small.v_new), d(small.k_cache), d(small.v_cache),
+                               d(small.block_table), d(small.q_start_loc), max_q_len=small.max_q,
+                               max_ctx_len=small.max_ctx, ranges=(d(rp), d(rs), d(rl), mr), k_scale=d(small.k_scale),
+                               v_scale=d(small.v_scale))
+    assert "row_blocks=5" not in pr.describe_plan(), pr.describe_plan()
+
+
 def test_fp8_codes_decode_like_torch(dev):
     """All 256 e4m3 codes through the kernel's dequantisation == torch.float8_e4m3fn -> float."""
     ops = _ops()
