@@ -262,40 +262,67 @@ __global__ __launch_bounds__(256) void evict_colsum_kernel(const float* __restri
 // above touch 128 bytes per row and keep few DRAM pages open); the per-head sums go to a workspace and
 // a second kernel adds the heads of a group in index order.  Same order of additions, same bits.
 constexpr int kHeadsumCols = 4;  // columns per thread at most
+// NCOL columns per thread (c0 + t + 256 j); a thread past the end of the range reads the range's last column again
+// and does not store.  No branch around a load: with one per load the kernel was bound by instruction issue.
+// The row's base address is uniform (scalar registers), the column a 32-bit byte offset per lane.
+template <int NCOL>
 __global__ __launch_bounds__(256) void evict_headsum_kernel(const float* __restrict__ probs, long n_heads, long n_q,
                                                             long n_keys, long width, float* __restrict__ hsum) {
   const long chunk = blockIdx.z, head = blockIdx.y;
   const long c0 = (long)blockIdx.x * width;
   long c1 = c0 + width;
   c1 = c1 < n_keys ? c1 : n_keys;
-  const float* p = probs + (chunk * n_heads + head) * n_q * n_keys;
-  float acc[kHeadsumCols];
-  long col[kHeadsumCols];
+  const char* p = reinterpret_cast<const char*>(probs + (chunk * n_heads + head) * n_q * n_keys + c0);
+  const unsigned last = (unsigned)(c1 - c0 - 1);
+  const long row_bytes = n_keys * 4;
+  float acc[NCOL];
+  unsigned off[NCOL];
 #pragma unroll
-  for (int j = 0; j < kHeadsumCols; ++j) {
+  for (int j = 0; j < NCOL; ++j) {
     acc[j] = 0.f;
-    const long c = c0 + threadIdx.x + 256L * j;
-    col[j] = c < c1 ? c : -1;
+    const unsigned c = threadIdx.x + 256u * j;
+    off[j] = (c < last ? c : last) * 4u;
   }
   long q = 0;
-  for (; q + 8 <= n_q; q += 8) {
-    float v[8][kHeadsumCols];
+  constexpr int R = 8;  // rows in flight (16: no faster)
+  for (; q + R <= n_q; q += R) {
+    float v[R][NCOL];
 #pragma unroll
-    for (int u = 0; u < 8; ++u)
+    for (int u = 0; u < R; ++u)
 #pragma unroll
-      for (int j = 0; j < kHeadsumCols; ++j) v[u][j] = col[j] >= 0 ? p[(q + u) * n_keys + col[j]] : 0.f;
+      for (int j = 0; j < NCOL; ++j) v[u][j] = *reinterpret_cast<const float*>(p + (q + u) * row_bytes + off[j]);
 #pragma unroll
-    for (int u = 0; u < 8; ++u)
+    for (int u = 0; u < R; ++u)
 #pragma unroll
-      for (int j = 0; j < kHeadsumCols; ++j) acc[j] += v[u][j];
+      for (int j = 0; j < NCOL; ++j) acc[j] += v[u][j];
   }
   for (; q < n_q; ++q)
 #pragma unroll
-    for (int j = 0; j < kHeadsumCols; ++j)
-      if (col[j] >= 0) acc[j] += p[q * n_keys + col[j]];
+    for (int j = 0; j < NCOL; ++j) acc[j] += *reinterpret_cast<const float*>(p + q * row_bytes + off[j]);
 #pragma unroll
-  for (int j = 0; j < kHeadsumCols; ++j)
-    if (col[j] >= 0) hsum[(chunk * n_heads + head) * n_keys + col[j]] = acc[j];
+  for (int j = 0; j < NCOL; ++j) {
+    const long c = c0 + threadIdx.x + 256L * j;
+    if (c < c1) hsum[(chunk * n_heads + head) * n_keys + c] = acc[j];
+  }
+}
+
+// Column ranges and launch of evict_headsum_kernel: enough workgroups for two per compute unit where the shape has
+// them, ranges of at most 256 * kHeadsumCols columns.
+static int launch_headsum(const float* probs, long n_chunks, long n_heads, long n_queries, long n_keys, float* hsum,
+                          hipStream_t st) {
+  long parts = (512 + n_heads * n_chunks - 1) / (n_heads * n_chunks);
+  const long min_parts = (n_keys + 256 * kHeadsumCols - 1) / (256 * kHeadsumCols);
+  parts = parts < min_parts ? min_parts : parts;
+  const long width = (n_keys + parts - 1) / parts;
+  parts = (n_keys + width - 1) / width;
+  const dim3 grid((unsigned)parts, (unsigned)n_heads, (unsigned)n_chunks);
+  switch ((width + 255) / 256) {
+    case 1: hipLaunchKernelGGL(evict_headsum_kernel<1>, grid, dim3(256), 0, st, probs, n_heads, n_queries, n_keys, width, hsum); break;
+    case 2: hipLaunchKernelGGL(evict_headsum_kernel<2>, grid, dim3(256), 0, st, probs, n_heads, n_queries, n_keys, width, hsum); break;
+    case 3: hipLaunchKernelGGL(evict_headsum_kernel<3>, grid, dim3(256), 0, st, probs, n_heads, n_queries, n_keys, width, hsum); break;
+    default: hipLaunchKernelGGL(evict_headsum_kernel<4>, grid, dim3(256), 0, st, probs, n_heads, n_queries, n_keys, width, hsum); break;
+  }
+  return launch_status();
 }
 
 __global__ __launch_bounds__(256) void evict_groupsum_kernel(const float* __restrict__ hsum, long n_heads, long hpg,
@@ -628,15 +655,8 @@ extern "C" int pdllm_evict_colsum(const float* probs, int64_t n_chunks, int64_t 
   if (workspace != nullptr && blocks64 < 1024 && n_heads <= 65535) {
     // few chunks: one workgroup per (chunk, head, column range), per-head sums through the workspace
     if (workspace_bytes < n_chunks * n_heads * n_keys * 4 || ((uintptr_t)workspace % 4)) return PDLLM_ERR_WORKSPACE;
-    long parts = (512 + n_heads * n_chunks - 1) / (n_heads * n_chunks);
-    const long min_parts = (n_keys + 256 * kHeadsumCols - 1) / (256 * kHeadsumCols);
-    parts = parts < min_parts ? min_parts : parts;
-    const long width = (n_keys + parts - 1) / parts;
-    parts = (n_keys + width - 1) / width;
     float* hsum = static_cast<float*>(workspace);
-    hipLaunchKernelGGL(evict_headsum_kernel, dim3((unsigned)parts, (unsigned)n_heads, (unsigned)n_chunks), dim3(256), 0,
-                       st, probs, (long)n_heads, (long)n_queries, (long)n_keys, width, hsum);
-    int rc = launch_status();
+    int rc = launch_headsum(probs, n_chunks, n_heads, n_queries, n_keys, hsum, st);
     if (rc != PDLLM_OK) return rc;
     hipLaunchKernelGGL(evict_groupsum_kernel,
                        dim3((unsigned)((n_keys + 255) / 256), (unsigned)(n_heads / heads_per_group), (unsigned)n_chunks),
@@ -681,15 +701,8 @@ extern "C" int pdllm_evict_keep_from_probs(const float* probs, int64_t n_chunks,
                                force_keep_first, indices_out, stream);
   }
   if (workspace_bytes < n_chunks * n_heads * n_keys * 4 || ((uintptr_t)workspace % 4)) return PDLLM_ERR_WORKSPACE;
-  long parts = (512 + n_heads * n_chunks - 1) / (n_heads * n_chunks);
-  const long min_parts = (n_keys + 256 * kHeadsumCols - 1) / (256 * kHeadsumCols);
-  parts = parts < min_parts ? min_parts : parts;
-  const long width = (n_keys + parts - 1) / parts;
-  parts = (n_keys + width - 1) / width;
   float* hsum = static_cast<float*>(workspace);
-  hipLaunchKernelGGL(evict_headsum_kernel, dim3((unsigned)parts, (unsigned)n_heads, (unsigned)n_chunks), dim3(256), 0,
-                     st, probs, (long)n_heads, (long)n_queries, (long)n_keys, width, hsum);
-  const int rc = launch_status();
+  const int rc = launch_headsum(probs, n_chunks, n_heads, n_queries, n_keys, hsum, st);
   if (rc != PDLLM_OK) return rc;
   hipLaunchKernelGGL(evict_groupsum_select_kernel, dim3((unsigned)(n_chunks * n_groups)), dim3(kSelThreads), 0, st,
                      hsum, (long)n_heads, (long)heads_per_group, (long)n_keys, (long)keep, keep_high ? 1 : 0,
