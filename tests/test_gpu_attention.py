@@ -331,6 +331,19 @@ def test_fp8_default_plan_takes_groups_of_five_where_they_fill(dev, q_len, Hq, H
     assert "row_blocks=5" not in pr.describe_plan(), pr.describe_plan()
 
 
+@pytest.mark.parametrize("plan", [dict(), dict(num_splits=1), dict(num_splits=4)], ids=["default", "unsplit", "split4"])
+def test_fp8_five_row_blocks_ragged_requests(dev, plan):
+    """The kernel with producer waves on requests of very different prefix lengths: one with a single chunk, one with
+    no visible key at all (its pieces hold tiles of the active block only, or nothing), one whose ranges end inside a
+    page; pieces past the end of a short request are empty."""
+    case = configs.chunked_prefix_case(83, n_req=4, n_chunks=6, chunk_tokens=330, topk=5, q_len=140, Hq=8, Hkv=8,
+                                       fp8=True, shared_prefix=False)
+    case.ranges[1] = case.ranges[1][:1]
+    case.ranges[2] = []
+    case.ranges[3] = [(s, l - 37) for s, l in case.ranges[3][:3]]
+    check(run_case(case, dev, rows_per_group=160, **plan), oracle_case(case))
+
+
 def test_fp8_codes_decode_like_torch(dev):
     """All 256 e4m3 codes through the kernel's dequantisation == torch.float8_e4m3fn -> float."""
     ops = _ops()
