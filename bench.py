@@ -318,6 +318,9 @@ def x_compact(torch, ops, dev, gd):
     g = torch.Generator().manual_seed(5)
     keep = [torch.stack([torch.randperm(n_tok, generator=g)[:kept].sort().values for _ in range(HKV)]).to(dev)
             for _ in range(layers)]
+    # (the engine hands the compaction what its normalisation step returned: fastdllm_engine.py:1940 -> 2081)
+    keep, _ = engine_ops.normalize_per_head_keep_indices(keep, num_layers=layers, num_heads=HKV, full_prompt_len=n_tok,
+                                                         device=dev)
     us = _time_us(torch, lambda: engine_ops.compact_prompt_cache_per_layer_per_head(kv, page_ids, keep), 3, 1)
     by = 2 * layers * HKV * kept * D * 2 * 2
     return {"us_per_request": us, **_hbm(by, us)}

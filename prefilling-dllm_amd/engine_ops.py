@@ -182,6 +182,24 @@ def compact_prompt_cache_per_head(layer_cache: torch.Tensor, page_ids: torch.Ten
     return active_len
 
 
+def _as_one_stack(tensors: Sequence[torch.Tensor], device) -> Optional[torch.Tensor]:
+    """The [L, H, n] tensor the given per-layer tensors are consecutive slices of, or None.  normalize_per_head_keep_indices
+    returns such slices (as the reference's engine passes the output of its _normalize_per_head_keep_indices on to
+    the compaction, ENG:1940 -> 2081): stacking them again would copy 28 tensors for nothing."""
+    first = tensors[0]
+    if not isinstance(first, torch.Tensor) or first.dtype != torch.long or first.device != torch.device(device) \
+            or first.dim() != 2 or not first.is_contiguous():
+        return None
+    step = first.numel()
+    store = first.untyped_storage().data_ptr()
+    for l, t in enumerate(tensors):
+        if (not isinstance(t, torch.Tensor) or t.dtype != torch.long or t.device != first.device or t.shape != first.shape
+                or not t.is_contiguous() or t.untyped_storage().data_ptr() != store
+                or t.storage_offset() != first.storage_offset() + l * step):
+            return None
+    return torch.as_strided(first, (len(tensors),) + tuple(first.shape), (step, first.shape[1], 1))
+
+
 def compact_prompt_cache_per_layer_per_head(kv_cache: torch.Tensor, prompt_page_ids: Sequence[int],
                                             keep_indices_per_layer_per_head: Sequence[torch.Tensor]) -> int:
     """_compact_prompt_cache_per_layer_per_head (ENG:607-638) on kv_cache [2, L, pages, P, Hkv, d]: all layers, K and
@@ -192,7 +210,9 @@ def compact_prompt_cache_per_layer_per_head(kv_cache: torch.Tensor, prompt_page_
     active_len = int(keep_indices_per_layer_per_head[0].shape[1])
     if active_len <= 0:
         return 0
-    keep = torch.stack([k.to(device=kv_cache.device, dtype=torch.long) for k in keep_indices_per_layer_per_head])
+    keep = _as_one_stack(keep_indices_per_layer_per_head, kv_cache.device)
+    if keep is None:
+        keep = torch.stack([k.to(device=kv_cache.device, dtype=torch.long) for k in keep_indices_per_layer_per_head])
     if kv_cache.is_contiguous() and keep.shape[0] == kv_cache.shape[1]:
         ops.kv_compact_per_head(kv_cache, page_ids, keep)
     else:       # a view of a larger cache, or fewer keep lists than layers: layer by layer

@@ -273,6 +273,22 @@ def test_page_pool_edge_cases():
     assert list(a.free_pages) == [3, 1, 0] and p == [0, 1, 2]
 
 
+def test_normalised_keep_indices_are_taken_as_one_stack():
+    """What normalize_per_head_keep_indices returns is a list of slices of one [L, H, n] tensor; the compaction
+    recognises that and uses the tensor as it is.  Anything else (copies, another order, another dtype) is stacked."""
+    import torch
+    from prefilling_dllm_amd.engine_ops import _as_one_stack, normalize_per_head_keep_indices as norm
+    given = [torch.randint(0, 50, (3, 7)) for _ in range(4)]
+    views, n = norm(given, num_layers=4, num_heads=3, full_prompt_len=50, device="cpu")
+    one = _as_one_stack(views, "cpu")
+    assert n == 7 and one is not None and one.shape == (4, 3, 7) and torch.equal(one, torch.stack(given))
+    assert one.data_ptr() == views[0].data_ptr()
+    assert _as_one_stack(given, "cpu") is None                                # separate tensors
+    assert _as_one_stack([views[1], views[0], views[2], views[3]], "cpu") is None   # not in layer order
+    assert _as_one_stack([v.to(torch.int32) for v in views], "cpu") is None
+    assert _as_one_stack([v.t() for v in views], "cpu") is None
+
+
 def test_normalize_per_head_keep_indices_contract():
     """_normalize_per_head_keep_indices (fastdllm_engine.py:560-605): one [heads, n] index tensor per layer, one
     common n, entries inside the prompt; the error names the first offending layer."""
